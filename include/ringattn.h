@@ -1,0 +1,158 @@
+/*
+ * ringattn.h -- C ABI of the MI355X (gfx950) ring-attention forward engine.
+ *
+ * Every entry point is extern "C", takes plain pointers and sizes, and returns an
+ * int status (0 = RINGATTN_OK).  Argument validation happens before the first HIP
+ * call, so bad arguments are reported on a host without a GPU as well.  Tensors
+ * are device-resident and contiguous, the convention of the reference's
+ * include/attention_api.cuh:12-18 (CHECK_CUDA / CHECK_CONTIGUOUS).  Where the
+ * reference prints and exits on an error (include/attention_api.cuh:20-29,
+ * csrc/utils.h:1-11), this library returns a code; ringattn_strerror() names it.
+ *
+ * Layout: Q, K, V, O are [batch, heads, S, dim] row-major, so each (batch, head)
+ * slab is the reference's [seqlen, dim] layout (csrc/ring_attention.cu:422-426).
+ * The sequence is split into npes chunks in order; virtual ring rank r owns rows
+ * [r*c, (r+1)*c).  At ring step s rank r works on KV chunk (r + s) mod npes
+ * (csrc/ring_attention.cu:463,531,615) -- by indexing, no data is moved.
+ */
+#ifndef RINGATTN_H
+#define RINGATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RINGATTN_OK 0
+#define RINGATTN_ERR_NULL 1        /* a required pointer is NULL */
+#define RINGATTN_ERR_NPES 2        /* npes < 1 or above RINGATTN_MAX_NPES */
+#define RINGATTN_ERR_DIM 3         /* dim not in {64, 128} */
+#define RINGATTN_ERR_DTYPE 4       /* dtype not fp16 / bf16 */
+#define RINGATTN_ERR_SEQLEN 5      /* chunk lengths not equal, not positive, or not a multiple of 128 */
+#define RINGATTN_ERR_SHAPE 6       /* batch or heads < 1, sizes overflow */
+#define RINGATTN_ERR_WORKSPACE 7   /* caller workspace missing or too small */
+#define RINGATTN_ERR_RANK 8        /* mype / step outside [0, npes) */
+#define RINGATTN_ERR_PLAN 9        /* plan handle invalid or already destroyed */
+#define RINGATTN_ERR_HIP 10        /* a HIP runtime call failed (see ringattn_last_hip_error) */
+#define RINGATTN_ERR_ALLOC 11      /* device or host allocation failed */
+#define RINGATTN_ERR_ALIGN 12      /* a tensor pointer is not 16-byte aligned */
+
+#define RINGATTN_DTYPE_FP16 0
+#define RINGATTN_DTYPE_BF16 1
+
+#define RINGATTN_MAX_NPES 64
+#define RINGATTN_TILE 128          /* chunk lengths must be multiples of this */
+
+#define RINGATTN_FLAG_GRAPH 1      /* capture the step loop + merge in a hipGraph and replay it */
+
+/*
+ * Replaces struct Ring_fwd_params (csrc/ring.h:5-19).  npes, h_seqlen, dim and
+ * softmax_scale keep their meaning; mype is gone because one call runs every
+ * virtual rank; the device copy of seqlen and the k/v staging buffers are gone
+ * because nothing is fetched from a peer.  batch, heads, dtype, causal are the
+ * generalisations the reference hard-wires (fp16, one head, non-causal:
+ * csrc/ring_attention.cu:18,422-426,530).
+ */
+typedef struct ringattn_params {
+  int npes;              /* P: virtual ring ranks */
+  const int* h_seqlen;   /* [npes] tokens per rank (host array, read during the call only) */
+  int dim;               /* head dimension: 64 or 128 */
+  float softmax_scale;   /* logit scale; <= 0 selects 1/sqrt(dim) */
+  int batch;
+  int heads;
+  int dtype;             /* RINGATTN_DTYPE_* of Q, K, V and O */
+  int causal;            /* 0: every rank sees every chunk; 1: chunks in sequence order, KV chunk j > r skipped, j == r masked */
+  int flags;             /* RINGATTN_FLAG_* */
+} ringattn_params;
+
+typedef struct ringattn_plan ringattn_plan;
+
+/* Bytes of device workspace a plan needs (per-step partial O and LSE for every ring
+ * step): npes * batch*heads*S * (dim + 1) * 4.  0 if the parameters are invalid. */
+size_t ringattn_workspace_bytes(const ringattn_params* params);
+
+/*
+ * Create a plan: validates the parameters and allocates the workspace ONCE -- the
+ * job set_params_fprop (csrc/ring_attention.cu:361-395) does on every call with a
+ * cudaMalloc and two nvshmem_mallocs that are never freed (:383-394).
+ * If workspace != NULL it is used instead of an internal allocation and must hold
+ * at least ringattn_workspace_bytes() bytes (workspace_bytes is checked).
+ */
+int ringattn_plan_create(const ringattn_params* params, void* workspace, size_t workspace_bytes,
+                         ringattn_plan** plan_out);
+
+/* Destroy a plan and free what it allocated.  NULL or an already destroyed plan gives RINGATTN_ERR_PLAN. */
+int ringattn_plan_destroy(ringattn_plan* plan);
+
+/*
+ * The whole forward for all npes virtual ranks: replaces ring_attention()
+ * (csrc/ring_attention.cu:706-722) run on every PE.  Step loop (one block-attention
+ * launch per ring step, all active ranks batched) followed by one npes-way merge.
+ *   q, k, v : [batch, heads, S, dim] dtype     out : same shape and dtype
+ *   lse     : [batch, heads, S] fp32, natural log (the reference never writes it)
+ * Asynchronous on `stream` (a hipStream_t, or NULL for the default stream); the
+ * reference blocks with cudaDeviceSynchronize (:721) -- callers that want that
+ * synchronise the stream.  A plan is used by one host thread at a time.
+ */
+int ringattn_fwd(ringattn_plan* plan, const void* q, const void* k, const void* v,
+                 void* out, float* lse, void* stream);
+
+/*
+ * One ring step (the body of the reference's step loop, csrc/ring_attention.cu:456-620,
+ * for every active rank at once): rank r attends KV chunk (r + step) mod npes and the
+ * normalised fp32 partial O [batch, heads, S, dim] and fp32 partial LSE
+ * [batch, heads, S] are written for the rows of the active ranks.  Rows of ranks that
+ * are inactive in this step (causal, chunk j > r) are left untouched.
+ */
+int ringattn_block_fwd(ringattn_plan* plan, int step, const void* q, const void* k, const void* v,
+                       float* o_part, float* lse_part, void* stream);
+
+/*
+ * Cross-step merge (no function of its own in the reference: it is the algebra of
+ * carrying max / sum / acc-O across steps, csrc/ring_attention.cu:207-245,621-633):
+ *   lse = logsumexp_s lse_parts[s];  out = sum_s exp(lse_parts[s] - lse) * o_parts[s]
+ * o_parts [n_parts, rows, dim] fp32, lse_parts [n_parts, rows] fp32 (a part with
+ * lse = -inf is the identity); out [rows, dim] dtype; lse [rows] fp32.
+ */
+int ringattn_merge(const float* o_parts, const float* lse_parts, int n_parts, int64_t rows, int dim,
+                   int dtype, void* out, float* lse, void* stream);
+
+/*
+ * Reference-shaped convenience entry: the signature of
+ *   void ring_attention(FPC* q, FPC* k, FPC* v, float* out, int npes, int mype,
+ *                       int* seqlen, int dim, int max_seq)   (csrc/ring_attention.cu:706)
+ * for ONE head and ONE rank: q is rank mype's [seqlen[mype], dim] block; k and v hold
+ * the chunks of all ranks back to back ([sum seqlen, dim]) -- what the reference
+ * reaches through NVSHMEM gets (:612-619); out is [seqlen[mype], dim] in `dtype`
+ * (the reference declares float* but stores 16-bit values, :635,763); lse (may be
+ * NULL) is [seqlen[mype]] fp32.  max_seq is accepted for signature parity and only
+ * checked (>= every seqlen).  Blocks until the result is ready, like the reference (:721).
+ */
+int ringattn_ring_attention(const void* q, const void* k, const void* v, void* out, float* lse,
+                            int npes, int mype, const int* seqlen, int dim, int max_seq,
+                            int dtype, int causal, float softmax_scale);
+
+/*
+ * Seeded input generator -- the counterpart of fillWithNum / initQKV
+ * (csrc/ring_attention.cu:731-748), which fill a host buffer and copy it to the
+ * device.  Writes n values of N(0, sigma^2), rounded to nearest-even into `dtype`,
+ * to a HOST buffer: element i uses counters 2*(offset+i)+1 and 2*(offset+i)+2 of the
+ * splitmix64 stream keyed by `seed` (Box-Muller, cosine branch).  Pure host code.
+ */
+int ringattn_fill_normal(void* dst_host, int dtype, int64_t n, uint64_t seed, int64_t offset, double sigma);
+
+/* The reference's own deterministic fill h[i*n+j] = i/130 + j/110 + i*j/600
+ * (csrc/ring_attention.cu:731-741), rounded into `dtype`, for an [m, n] host matrix. */
+int ringattn_fill_reference_pattern(void* dst_host, int dtype, int m, int n);
+
+const char* ringattn_strerror(int code);
+
+/* The hipError_t (as int) of the last failing HIP call seen by this thread, 0 if none. */
+int ringattn_last_hip_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RINGATTN_H */

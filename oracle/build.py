@@ -1,0 +1,32 @@
+"""Builds the CPU oracle (test infrastructure, never part of the product path).
+
+  oracle/liboracle.so       <- oracle/attention_oracle.c   (gcc -O3 -fopenmp)
+
+The reference's own path cannot be compiled here: csrc/ring_attention.cu needs nvcc,
+CUTLASS/CuTe (an empty, un-fetched submodule) and NVSHMEM, and the file is truncated
+(csrc/ring_attention.cu:244-248), so there is no oracle/_ref build.
+"""
+import os
+import shutil
+import subprocess
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "liboracle.so")
+
+
+def build_oracle():
+    gcc = shutil.which("gcc")
+    if not gcc:
+        raise RuntimeError("gcc not found: cannot build the oracle")
+    tmp = LIB_PATH + ".tmp"
+    cmd = [gcc, "-O3", "-march=x86-64-v3", "-fopenmp", "-fPIC", "-shared", "-std=c11",
+           os.path.join(HERE, "attention_oracle.c"), "-o", tmp, "-lm"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("gcc failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_oracle())

@@ -1,0 +1,162 @@
+"""Host-side mirror of the reference's entry points on top of the C ABI.
+
+`RingAttention` is a plan (parameters + workspace, created once) with `forward`,
+`block_forward` and `merge` methods; `ring_attention` has the reference's
+`ring_attention(q, k, v, out, npes, mype, seqlen, dim, max_seq)` argument list
+(csrc/ring_attention.cu:706).  torch is used only to own device memory and to name
+the stream; every computation goes through libringattn.so.
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib
+from ._lib import RingattnParams, check
+
+DTYPE_CODE = {"fp16": 0, "bf16": 1, torch.float16: 0, torch.bfloat16: 1}
+TORCH_DTYPE = {0: torch.float16, 1: torch.bfloat16}
+FLAG_GRAPH = 1
+
+
+def _stream_ptr(stream=None):
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _check_tensor(t, name, dtype=None):
+    # conventions of include/attention_api.cuh:12-18: device-resident and contiguous
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a device tensor")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise ValueError(f"{name} must have dtype {dtype}")
+
+
+def make_params(npes, seqlen, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, flags=0):
+    arr = (ctypes.c_int * len(seqlen))(*[int(x) for x in seqlen])
+    p = RingattnParams(int(npes), ctypes.cast(arr, _lib.c_int_p), int(dim), float(softmax_scale), int(batch),
+                       int(heads), DTYPE_CODE[dtype], int(bool(causal)), int(flags))
+    p._keepalive = arr
+    return p
+
+
+class RingAttention:
+    """A forward plan for P virtual ring ranks on one GPU."""
+
+    def __init__(self, npes, chunk, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, graph=False):
+        self.lib = _lib.load()
+        self.npes, self.chunk, self.dim, self.batch, self.heads = npes, chunk, dim, batch, heads
+        self.dtype_code = DTYPE_CODE[dtype]
+        self.torch_dtype = TORCH_DTYPE[self.dtype_code]
+        self.causal = bool(causal)
+        self.seq = npes * chunk
+        self.params = make_params(npes, [chunk] * npes, dim, batch, heads, dtype, causal, softmax_scale,
+                                  FLAG_GRAPH if graph else 0)
+        self.handle = ctypes.c_void_p()
+        check(self.lib.ringattn_plan_create(ctypes.byref(self.params), None, 0, ctypes.byref(self.handle)),
+              "ringattn_plan_create")
+
+    def close(self):
+        if self.handle:
+            check(self.lib.ringattn_plan_destroy(self.handle), "ringattn_plan_destroy")
+            self.handle = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _shape(self):
+        return (self.batch, self.heads, self.seq, self.dim)
+
+    def forward(self, q, k, v, out=None, lse=None, stream=None):
+        for t, nm in ((q, "q"), (k, "k"), (v, "v")):
+            _check_tensor(t, nm, self.torch_dtype)
+            if tuple(t.shape) != self._shape():
+                raise ValueError(f"{nm} must have shape {self._shape()}")
+        if out is None:
+            out = torch.empty_like(q)
+        if lse is None:
+            lse = torch.empty((self.batch, self.heads, self.seq), dtype=torch.float32, device=q.device)
+        _check_tensor(out, "out", self.torch_dtype)
+        _check_tensor(lse, "lse", torch.float32)
+        check(self.lib.ringattn_fwd(self.handle, _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _stream_ptr(stream)),
+              "ringattn_fwd")
+        return out, lse
+
+    def block_forward(self, step, q, k, v, o_part=None, lse_part=None, stream=None):
+        for t, nm in ((q, "q"), (k, "k"), (v, "v")):
+            _check_tensor(t, nm, self.torch_dtype)
+        if o_part is None:
+            o_part = torch.zeros(self._shape(), dtype=torch.float32, device=q.device)
+        if lse_part is None:
+            lse_part = torch.full((self.batch, self.heads, self.seq), float("-inf"), dtype=torch.float32, device=q.device)
+        check(self.lib.ringattn_block_fwd(self.handle, int(step), _ptr(q), _ptr(k), _ptr(v), _ptr(o_part),
+                                          _ptr(lse_part), _stream_ptr(stream)), "ringattn_block_fwd")
+        return o_part, lse_part
+
+
+def merge(o_parts, lse_parts, dtype, stream=None):
+    """n-way (O, LSE) merge.  o_parts [n, rows, d] fp32, lse_parts [n, rows] fp32."""
+    lib = _lib.load()
+    _check_tensor(o_parts, "o_parts", torch.float32)
+    _check_tensor(lse_parts, "lse_parts", torch.float32)
+    n, rows, d = o_parts.shape
+    code = DTYPE_CODE[dtype]
+    out = torch.empty((rows, d), dtype=TORCH_DTYPE[code], device=o_parts.device)
+    lse = torch.empty((rows,), dtype=torch.float32, device=o_parts.device)
+    check(lib.ringattn_merge(_ptr(o_parts), _ptr(lse_parts), n, rows, d, code, _ptr(out), _ptr(lse), _stream_ptr(stream)),
+          "ringattn_merge")
+    return out, lse
+
+
+def ring_attention(q, k, v, out, npes, mype, seqlen, dim, max_seq, lse=None, causal=False, softmax_scale=0.0):
+    """Reference-shaped call (csrc/ring_attention.cu:706): one head, rank `mype` only.
+
+    q [seqlen[mype], dim] is the rank's block, k / v [sum(seqlen), dim] hold all ranks'
+    chunks, out [seqlen[mype], dim].  Blocks until done, like the reference (:721).
+    """
+    lib = _lib.load()
+    for t, nm in ((q, "q"), (k, "k"), (v, "v"), (out, "out")):
+        _check_tensor(t, nm, q.dtype)
+    arr = (ctypes.c_int * len(seqlen))(*[int(x) for x in seqlen])
+    check(lib.ringattn_ring_attention(_ptr(q), _ptr(k), _ptr(v), _ptr(out),
+                                      _ptr(lse) if lse is not None else None, int(npes), int(mype), arr, int(dim),
+                                      int(max_seq), DTYPE_CODE[q.dtype], int(bool(causal)), float(softmax_scale)),
+          "ringattn_ring_attention")
+    return out
+
+
+# ---- seeded inputs (counterpart of fillWithNum / initQKV, csrc/ring_attention.cu:731-748) ----
+
+def fill_normal(n, dtype, seed, offset=0, sigma=1.0):
+    """n values of N(0, sigma^2) rounded into `dtype`, as a uint16 numpy array of bit patterns."""
+    lib = _lib.load()
+    buf = np.empty(int(n), dtype=np.uint16)
+    check(lib.ringattn_fill_normal(buf.ctypes.data_as(ctypes.c_void_p), DTYPE_CODE[dtype], int(n), int(seed), int(offset),
+                                   float(sigma)), "ringattn_fill_normal")
+    return buf
+
+
+def make_qkv_bits(w):
+    """Q, K, V of a Workload as uint16 bit patterns [B, H, S, d]; stream order Q, K, V."""
+    n = w.batch * w.heads * w.seq * w.dim
+    shape = (w.batch, w.heads, w.seq, w.dim)
+    q = fill_normal(n, w.dtype, w.seed, 0, w.sigma_qk).reshape(shape)
+    k = fill_normal(n, w.dtype, w.seed, n, w.sigma_qk).reshape(shape)
+    v = fill_normal(n, w.dtype, w.seed, 2 * n, w.sigma_v).reshape(shape)
+    return q, k, v
+
+
+def bits_to_tensor(bits, dtype, device="cuda"):
+    """uint16 bit patterns -> torch tensor of the 16-bit float dtype on `device`."""
+    t = torch.from_numpy(bits.view(np.int16)).view(TORCH_DTYPE[DTYPE_CODE[dtype]])
+    return t.to(device)
