@@ -1,0 +1,159 @@
+"""Headline benchmark: ring-attention forward on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4]
+
+A step is one full forward of the workload: the ring step loop (one block-attention
+launch per ring step) plus the P-way merge, with Q/K/V already resident in HBM.  Prints
+one JSON line.  `value` is algorithmic TFLOP/s (4*B*H*d*visible (q,k) pairs per forward)
+over the wall time of K steps; `roofline` prices the block-attention kernel alone
+against the dense MFMA peak, timed with events on the launch stream in a separate
+pass; `merge` does the same for the merge kernel against HBM bandwidth; `cpu_baseline`
+is the CPU oracle timed on this host on a bounded sample of the same workload's rows.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# Published MI355X dense peaks used for the roofline (not the 2:1-sparsity figures)
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0}
+PEAK_HBM_GBS = 8000.0
+# HBM bytes per block-kernel launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
+# see profiles/; None where not measured for that workload.
+MEASURED_TRAFFIC = {}
+
+
+def describe(w):
+    return (f"{w.name}: {'causal' if w.causal else 'non-causal'} fwd, B={w.batch} H={w.heads} d={w.dim}, "
+            f"{w.npes} virtual ranks x {w.chunk} tokens (S={w.seq}), {w.dtype}, N(0,{w.sigma_qk:g}^2) Q/K seed {w.seed}")
+
+
+def pair_counts(w):
+    """(q, k) pairs visible in each ring step's launch."""
+    P, c = w.npes, w.chunk
+    out = []
+    for s in range(P):
+        if not w.causal:
+            out.append(P * c * c)
+        elif s == 0:
+            out.append(P * c * (c + 1) // 2)
+        else:
+            out.append(s * c * c)
+    return [x * w.batch * w.heads for x in out]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg4")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the cpu_baseline sample (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (P virtual ring ranks on one MI355X); use --gpus 1")
+
+    import numpy as np
+    import torch
+    from ringattention_amd import WORKLOADS, _lib, api
+    _lib.load()   # fails loudly if the HIP extension is missing
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    torch.cuda.set_device(0)
+    w = WORKLOADS[args.workload]
+
+    q, k, v = api.make_qkv_bits(w)
+    qd, kd, vd = (api.bits_to_tensor(x, w.dtype) for x in (q, k, v))
+    plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=w.graph)
+    out = torch.empty_like(qd)
+    lse = torch.empty((w.batch, w.heads, w.seq), dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream()
+
+    for _ in range(args.warmup):
+        plan.forward(qd, kd, vd, out, lse, stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        plan.forward(qd, kd, vd, out, lse, stream)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    tflops = w.flops / (ms_per_step * 1e-3) / 1e12
+
+    # ---- per-kernel pass: events on the launch stream around each block launch and the merge
+    eager = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=False)
+    o_parts = torch.empty((w.npes, w.batch, w.heads, w.seq, w.dim), dtype=torch.float32, device="cuda")
+    l_parts = torch.empty((w.npes, w.batch, w.heads, w.seq), dtype=torch.float32, device="cuda")
+    reps = max(3, min(args.steps, 10))
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(w.npes + 2)] for _ in range(reps)]
+    for rep in range(-1, reps):   # rep -1 warms up
+        for s in range(w.npes):
+            if rep >= 0:
+                ev[rep][s].record(stream)
+            eager.block_forward(s, qd, kd, vd, o_parts[s], l_parts[s], stream)
+        if rep >= 0:
+            ev[rep][w.npes].record(stream)
+        eager.merge_ring(o_parts, l_parts, out, lse, stream)
+        if rep >= 0:
+            ev[rep][w.npes + 1].record(stream)
+    torch.cuda.synchronize()
+    block_ms = [np.mean([ev[r][s].elapsed_time(ev[r][s + 1]) for r in range(reps)]) for s in range(w.npes)]
+    merge_ms = float(np.mean([ev[r][w.npes].elapsed_time(ev[r][w.npes + 1]) for r in range(reps)]))
+    pairs = pair_counts(w)
+    launch_flops = [4.0 * w.dim * p for p in pairs]
+    block_tflops = sum(launch_flops) / (sum(block_ms) * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[w.dtype]
+    roofline = {
+        "kernel": "block_attention_kernel", "bound": "mfma",
+        "achieved": round(block_tflops, 2), "peak": peak, "unit": "TFLOP/s", "frac": round(block_tflops / peak, 4),
+        "traffic": MEASURED_TRAFFIC.get(w.name),
+        "launches_per_step": w.npes, "avg_launch_ms": round(float(np.mean(block_ms)), 4),
+        "avg_launch_flop": float(np.mean(launch_flops)),
+    }
+    # merge: algorithmic bytes = active parts * (4 d + 4) read + (2 d + 4) written, per row
+    P = w.npes
+    parts_per_rank = [(r + 1) if w.causal else P for r in range(P)]
+    merge_bytes = w.batch * w.heads * w.chunk * sum(n * (4 * w.dim + 4) + 2 * w.dim + 4 for n in parts_per_rank)
+    merge = {"kernel": "merge_kernel", "bound": "hbm", "achieved": round(merge_bytes / (merge_ms * 1e-3) / 1e9, 1),
+             "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(merge_bytes / (merge_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+             "ms": round(merge_ms, 4), "bytes": merge_bytes}
+    eager.close()
+    plan.close()
+
+    # ---- CPU baseline: the oracle (a port; the reference has no CPU attention path) on a
+    # bounded, seeded sample of rows of the same workload
+    cpu = None
+    if args.cpu_seconds > 0:
+        from oracle import oracle
+        rng = np.random.default_rng(12345)
+        per_row = 4.0 * w.dim * (np.arange(w.seq) + 1 if w.causal else np.full(w.seq, w.seq))   # FLOP per row index
+        n, dt = 2048, 0.0
+        for _ in range(4):   # grow the sample until it costs about --cpu-seconds of CPU work
+            rows = rng.integers(0, w.rows, n)
+            t = time.perf_counter()
+            oracle.attention_rows(q, k, v, w.dtype, causal=w.causal, rows=rows)
+            dt = time.perf_counter() - t
+            if dt >= 0.6 * args.cpu_seconds or n >= w.rows:
+                break
+            n = int(min(w.rows, n * min(32.0, args.cpu_seconds / max(dt, 1e-3))))
+        fl = float(per_row[rows % w.seq].sum())
+        cpu = {"value": round(fl / dt / 1e12, 5), "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+               "sample": f"{n} seeded random query rows of {w.name} ({fl:.3e} FLOP) in {dt:.1f} s, fp64 oracle; "
+                         f"full forward extrapolates to {w.flops / (fl / dt):.0f} s"}
+
+    print(json.dumps({
+        "metric": "ring-attn fwd TFLOP/s + % bf16 MFMA peak, S=32K d=128 8-step ring, 1 GPU",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": w.dtype, "data": "synthetic",
+        "config": {"workload": describe(w), "algorithmic_flop": w.flops, "graph": bool(w.graph)},
+        "pct_mfma_peak": round(100.0 * tflops / peak, 2),
+        "roofline": roofline, "merge": merge, "cpu_baseline": cpu,
+    }))
+
+
+if __name__ == "__main__":
+    main()

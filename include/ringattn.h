@@ -120,6 +120,17 @@ int ringattn_merge(const float* o_parts, const float* lse_parts, int n_parts, in
                    int dtype, void* out, float* lse, void* stream);
 
 /*
+ * The merge as ringattn_fwd runs it, on caller-held partials: o_parts
+ * [npes, batch*heads*S, dim] and lse_parts [npes, batch*heads*S] as written by
+ * ringattn_block_fwd for steps 0..npes-1.  With a causal plan, part s of a row of rank r
+ * is read only if rank r was active in step s (s == 0 or r + s >= npes), so parts the
+ * step loop never wrote are never touched.  Like ringattn_merge, it has no counterpart
+ * function in the reference (csrc/ring_attention.cu:207-245,621-633 pin the algebra).
+ */
+int ringattn_merge_ring(ringattn_plan* plan, const float* o_parts, const float* lse_parts,
+                        void* out, float* lse, void* stream);
+
+/*
  * Reference-shaped convenience entry: the signature of
  *   void ring_attention(FPC* q, FPC* k, FPC* v, float* out, int npes, int mype,
  *                       int* seqlen, int dim, int max_seq)   (csrc/ring_attention.cu:706)

@@ -89,6 +89,7 @@ def attention_rows(q, k, v, dtype, causal=False, scale=None, rows=None):
 
     q, k, v: uint16 [B, H, S, d].  Returns (O [n, d] f64, LSE [n] f64)."""
     q, k, v = _u16(q), _u16(k), _u16(v)
+    assert q.shape == k.shape == v.shape, "q, k, v must have the same [B, H, S, d] shape"
     B, H, S, d = q.shape
     scale = default_scale(d) if scale is None else scale
     if rows is None:

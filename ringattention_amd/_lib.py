@@ -40,6 +40,7 @@ SYMBOLS = {
     "ringattn_block_fwd": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 6),
     "ringattn_merge": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
                                       ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
+    "ringattn_merge_ring": (ctypes.c_int, [ctypes.c_void_p] * 6),
     "ringattn_ring_attention": (ctypes.c_int, [ctypes.c_void_p] * 5 + [ctypes.c_int, ctypes.c_int, c_int_p,
                                                                        ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                                        ctypes.c_int, ctypes.c_float]),

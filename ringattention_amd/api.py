@@ -104,6 +104,19 @@ class RingAttention:
         return o_part, lse_part
 
 
+    def merge_ring(self, o_parts, lse_parts, out=None, lse=None, stream=None):
+        """Ring-aware merge of caller-held per-step partials [npes, B, H, S, d] / [npes, B, H, S]."""
+        _check_tensor(o_parts, "o_parts", torch.float32)
+        _check_tensor(lse_parts, "lse_parts", torch.float32)
+        if out is None:
+            out = torch.empty(self._shape(), dtype=self.torch_dtype, device=o_parts.device)
+        if lse is None:
+            lse = torch.empty((self.batch, self.heads, self.seq), dtype=torch.float32, device=o_parts.device)
+        check(self.lib.ringattn_merge_ring(self.handle, _ptr(o_parts), _ptr(lse_parts), _ptr(out), _ptr(lse),
+                                           _stream_ptr(stream)), "ringattn_merge_ring")
+        return out, lse
+
+
 def merge(o_parts, lse_parts, dtype, stream=None):
     """n-way (O, LSE) merge.  o_parts [n, rows, d] fp32, lse_parts [n, rows] fp32."""
     lib = _lib.load()

@@ -131,6 +131,24 @@ int launch_step(const ringattn_plan* pl, int s, const void* q, const void* k, co
   return RINGATTN_OK;
 }
 
+int launch_ring_merge(const ringattn_plan* pl, const float* o_parts, const float* lse_parts, void* out,
+                      float* lse, hipStream_t stream) {
+  ringattn::MergeArgs m;
+  m.o_parts = o_parts;
+  m.lse_parts = lse_parts;
+  m.out = out;
+  m.lse = lse;
+  m.rows = pl->d.rows;
+  m.part_stride_rows = pl->d.rows;
+  m.n_parts = pl->p.npes;
+  m.causal_ring = pl->p.causal ? 1 : 0;
+  m.S = (int)pl->d.S;
+  m.chunk = pl->d.chunk;
+  m.P = pl->p.npes;
+  RA_HIP(ringattn::launch_merge(m, pl->p.dtype, pl->p.dim, stream));
+  return RINGATTN_OK;
+}
+
 // The ring step loop (csrc/ring_attention.cu:456-620 moved to the host) plus the merge.
 int run_forward(const ringattn_plan* pl, const void* q, const void* k, const void* v, void* out,
                 float* lse, hipStream_t stream) {
@@ -140,20 +158,7 @@ int run_forward(const ringattn_plan* pl, const void* q, const void* k, const voi
                          pl->lse_parts + (size_t)s * pl->d.rows, stream);
     if (rc != RINGATTN_OK) return rc;
   }
-  ringattn::MergeArgs m;
-  m.o_parts = pl->o_parts;
-  m.lse_parts = pl->lse_parts;
-  m.out = out;
-  m.lse = lse;
-  m.rows = pl->d.rows;
-  m.part_stride_rows = pl->d.rows;
-  m.n_parts = P;
-  m.causal_ring = pl->p.causal ? 1 : 0;
-  m.S = (int)pl->d.S;
-  m.chunk = pl->d.chunk;
-  m.P = P;
-  RA_HIP(ringattn::launch_merge(m, pl->p.dtype, pl->p.dim, stream));
-  return RINGATTN_OK;
+  return launch_ring_merge(pl, pl->o_parts, pl->lse_parts, out, lse, stream);
 }
 
 void drop_graph(ringattn_plan* pl) {
@@ -282,6 +287,14 @@ int ringattn_block_fwd(ringattn_plan* plan, int step, const void* q, const void*
   if (step < 0 || step >= plan->p.npes) return RINGATTN_ERR_RANK;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o_part) || ((uintptr_t)lse_part & 3u)) return RINGATTN_ERR_ALIGN;
   return launch_step(plan, step, q, k, v, o_part, lse_part, (hipStream_t)stream);
+}
+
+int ringattn_merge_ring(ringattn_plan* plan, const float* o_parts, const float* lse_parts, void* out,
+                        float* lse, void* stream) {
+  if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
+  if (!o_parts || !lse_parts || !out || !lse) return RINGATTN_ERR_NULL;
+  if (!aligned16(o_parts) || !aligned16(out) || ((uintptr_t)lse_parts & 3u) || ((uintptr_t)lse & 3u)) return RINGATTN_ERR_ALIGN;
+  return launch_ring_merge(plan, o_parts, lse_parts, out, lse, (hipStream_t)stream);
 }
 
 int ringattn_merge(const float* o_parts, const float* lse_parts, int n_parts, int64_t rows, int dim,

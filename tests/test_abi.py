@@ -1,0 +1,130 @@
+"""The C ABI without a GPU: every symbol declared in include/ringattn.h is exported, and
+argument validation (which precedes every HIP call) returns the documented codes."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from ringattention_amd import _lib
+from ringattention_amd._lib import RingattnParams
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+OK, E_NULL, E_NPES, E_DIM, E_DTYPE, E_SEQLEN, E_SHAPE, E_WS, E_RANK, E_PLAN, E_HIP, E_ALLOC, E_ALIGN = range(13)
+
+
+def params(npes=2, seqlen=(128, 128), dim=64, batch=1, heads=1, dtype=0, causal=0, flags=0, scale=0.0):
+    arr = (ctypes.c_int * max(1, len(seqlen)))(*seqlen)
+    p = RingattnParams(npes, ctypes.cast(arr, _lib.c_int_p), dim, scale, batch, heads, dtype, causal, flags)
+    p._keep = arr
+    return p
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "ringattn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ringattn_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(ralib):
+    names = declared_functions()
+    assert len(names) >= 11
+    for n in names:
+        assert hasattr(ralib, n), f"{n} declared in ringattn.h but not exported"
+    assert set(names) == set(_lib.SYMBOLS), "ctypes binding and header disagree"
+
+
+def test_header_constants_match_error_strings(ralib):
+    text = open(os.path.join(ROOT, "include", "ringattn.h")).read()
+    codes = {k: int(v) for k, v in re.findall(r"#define (RINGATTN_(?:OK|ERR_[A-Z]+)) (\d+)", text)}
+    assert codes["RINGATTN_OK"] == 0 and codes["RINGATTN_ERR_ALIGN"] == E_ALIGN and len(codes) == 13
+    msgs = [ralib.ringattn_strerror(c).decode() for c in range(13)]
+    assert len(set(msgs)) == 13 and "unknown" in ralib.ringattn_strerror(99).decode()
+
+
+def test_parameter_validation(ralib):
+    wb = ralib.ringattn_workspace_bytes
+    assert wb(ctypes.byref(params())) == 2 * 256 * 65 * 4
+    h = ctypes.c_void_p()
+
+    def create(p):
+        return ralib.ringattn_plan_create(ctypes.byref(p) if p is not None else None, None, 0, ctypes.byref(h))
+
+    assert create(None) == E_NULL
+    assert ralib.ringattn_plan_create(ctypes.byref(params()), None, 0, None) == E_NULL
+    assert create(params(npes=0)) == E_NPES
+    assert create(params(npes=-3)) == E_NPES
+    assert create(params(npes=65, seqlen=(128,) * 65)) == E_NPES
+    p = params()
+    p.h_seqlen = None
+    assert create(p) == E_NULL
+    for bad_dim in (0, 32, 96, 256):
+        assert create(params(dim=bad_dim)) == E_DIM
+    assert create(params(dtype=2)) == E_DTYPE
+    assert create(params(dtype=-1)) == E_DTYPE
+    assert create(params(seqlen=(128, 256))) == E_SEQLEN      # unequal chunks
+    assert create(params(seqlen=(100, 100))) == E_SEQLEN      # not a multiple of the tile
+    assert create(params(seqlen=(0, 0))) == E_SEQLEN
+    assert create(params(seqlen=(-128, -128))) == E_SEQLEN
+    assert create(params(batch=0)) == E_SHAPE
+    assert create(params(heads=-1)) == E_SHAPE
+    assert create(params(scale=float("nan"))) == E_SHAPE
+    for bad in (params(npes=0), params(dim=7), params(seqlen=(64, 64))):
+        assert wb(ctypes.byref(bad)) == 0
+    assert wb(None) == 0
+
+
+def test_plan_lifetime_with_caller_workspace(ralib):
+    # a caller-provided workspace needs no HIP call, so the plan life cycle runs on a CPU host
+    p = params()
+    need = ralib.ringattn_workspace_bytes(ctypes.byref(p))
+    ws = np.zeros(need // 4 + 8, dtype=np.float32)
+    base = ws.ctypes.data + (-ws.ctypes.data % 16)
+    h = ctypes.c_void_p()
+    assert ralib.ringattn_plan_create(ctypes.byref(p), ctypes.c_void_p(base), need - 1, ctypes.byref(h)) == E_WS
+    assert ralib.ringattn_plan_create(ctypes.byref(p), ctypes.c_void_p(base + 4), need, ctypes.byref(h)) == E_ALIGN
+    assert ralib.ringattn_plan_create(ctypes.byref(p), ctypes.c_void_p(base), need, ctypes.byref(h)) == OK
+    assert h.value
+    # argument checks of the compute entry points come before any HIP work
+    x = ctypes.c_void_p(base)
+    assert ralib.ringattn_fwd(h, None, x, x, x, x, None) == E_NULL
+    assert ralib.ringattn_fwd(h, x, x, x, x, None, None) == E_NULL
+    assert ralib.ringattn_fwd(h, ctypes.c_void_p(base + 2), x, x, x, x, None) == E_ALIGN
+    assert ralib.ringattn_block_fwd(h, 2, x, x, x, x, x, None) == E_RANK
+    assert ralib.ringattn_block_fwd(h, -1, x, x, x, x, x, None) == E_RANK
+    assert ralib.ringattn_block_fwd(h, 0, x, x, None, x, x, None) == E_NULL
+    assert ralib.ringattn_plan_destroy(h) == OK
+    assert ralib.ringattn_plan_destroy(h) == E_PLAN          # double destroy
+    assert ralib.ringattn_fwd(h, x, x, x, x, x, None) == E_PLAN  # use after destroy
+    assert ralib.ringattn_plan_destroy(None) == E_PLAN
+
+
+def test_merge_and_reference_entry_validation(ralib):
+    buf = np.zeros(4096, dtype=np.float32)
+    x = ctypes.c_void_p(buf.ctypes.data + (-buf.ctypes.data % 16))
+    m = ralib.ringattn_merge
+    assert m(None, x, 2, 8, 64, 0, x, x, None) == E_NULL
+    assert m(x, x, 0, 8, 64, 0, x, x, None) == E_NPES
+    assert m(x, x, 2, 8, 48, 0, x, x, None) == E_DIM
+    assert m(x, x, 2, 8, 64, 5, x, x, None) == E_DTYPE
+    assert m(x, x, 2, -1, 64, 0, x, x, None) == E_SHAPE
+    ra = ralib.ringattn_ring_attention
+    sl = (ctypes.c_int * 2)(128, 128)
+    assert ra(x, x, x, x, None, 2, 2, sl, 64, 128, 0, 0, 0.0) == E_RANK
+    assert ra(x, x, x, x, None, 2, -1, sl, 64, 128, 0, 0, 0.0) == E_RANK
+    assert ra(x, x, x, x, None, 2, 0, sl, 64, 64, 0, 0, 0.0) == E_SEQLEN   # max_seq below a chunk
+    assert ra(None, x, x, x, None, 2, 0, sl, 64, 128, 0, 0, 0.0) == E_NULL
+    assert ra(x, x, x, x, None, 2, 0, sl, 80, 128, 0, 0, 0.0) == E_DIM
+    assert ra(x, x, x, x, None, 0, 0, sl, 64, 128, 0, 0, 0.0) == E_NPES
+    f = ralib.ringattn_fill_normal
+    assert f(None, 0, 4, 0, 0, 1.0) == E_NULL
+    assert f(x, 3, 4, 0, 0, 1.0) == E_DTYPE
+    assert f(x, 0, -4, 0, 0, 1.0) == E_SHAPE
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libringattn.so"))
+    with pytest.raises(RuntimeError, match="has not been built"):
+        _lib.load()
