@@ -53,6 +53,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg4")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the cpu_baseline sample (0 = skip)")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
+                    help="only run a plain device copy of MIB mebibytes a few times and exit: the known-size kernel "
+                         "that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (P virtual ring ranks on one MI355X); use --gpus 1")
@@ -64,6 +67,14 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     torch.cuda.set_device(0)
+    if args.copy_probe > 0:
+        src = torch.empty(args.copy_probe << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_probe_bytes": args.copy_probe << 20, "copies": 5}))
+        return
     w = WORKLOADS[args.workload]
 
     q, k, v = api.make_qkv_bits(w)

@@ -177,43 +177,41 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
 #pragma unroll
     for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
 
-  auto issue_tile = [&](int t, int buf) {
+  // direct-to-LDS loads of one K or V tile (this wave's share)
+  auto issue_k = [&](int t, int buf) {
     const char* kt = kbase + (int64_t)t * TILE;
-    const char* vt = vbase + (int64_t)t * TILE;
     const unsigned kd = __builtin_amdgcn_readfirstlane(smem_base + buf * TILE + wave * (LD_PER_WAVE * 1024));
-    const unsigned vd = kd + 2 * TILE;
 #pragma unroll
-    for (int i = 0; i < LD_PER_WAVE; ++i) {
-      load_lds_16(kt, goff_k[i], kd + i * 1024);
-      load_lds_16(vt, goff_v[i], vd + i * 1024);
-    }
+    for (int i = 0; i < LD_PER_WAVE; ++i) load_lds_16(kt, goff_k[i], kd + i * 1024);
   };
-
-  // Retire the Q loads here, with a wait the compiler can see: otherwise it places
-  // counted vmcnt waits at their first use inside the loop, and those would also
-  // drain the direct-to-LDS prefetch it does not know about.
-  __builtin_amdgcn_s_waitcnt(0);
-  issue_tile(0, 0);
-  for (int t = 0; t < n_tiles; ++t) {
-    const int buf = t & 1;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();  // tile t is in LDS; every wave is done with tile t-1
-    if (t + 1 < n_tiles) issue_tile(t + 1, buf ^ 1);
+  auto issue_v = [&](int t, int buf) {
+    const char* vt = vbase + (int64_t)t * TILE;
+    const unsigned vd = __builtin_amdgcn_readfirstlane(smem_base + (2 + buf) * TILE + wave * (LD_PER_WAVE * 1024));
+#pragma unroll
+    for (int i = 0; i < LD_PER_WAVE; ++i) load_lds_16(vt, goff_v[i], vd + i * 1024);
+  };
+  // K fragments (A operand of S^T = K Q^T) of a whole tile, LDS -> registers
+  s16x8 kf[KS][KB];
+  auto load_k_frags = [&](int buf) {
     const unsigned char* ks_lds = smem + buf * TILE;
-    const unsigned char* vs_lds = smem + (2 + buf) * TILE;
-
-    // S^T = K Q^T : keys x queries, fp32 accumulate (csrc/ring_attention.cu:565)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) kf[ks][kb] = *(const s16x8*)(ks_lds + kb * 32 * ROWB + koff[ks]);
+  };
+  // S^T = K Q^T : keys x queries, fp32 accumulate (csrc/ring_attention.cu:565), then the
+  // online softmax (:194-245).  Leaves P^T, rounded to the storage type, in pf as B operands.
+  s16x8 pf[KB][2];
+  auto scores_and_softmax = [&](int t) {
     f32x16 sacc[KB];
 #pragma unroll
-    for (int kb = 0; kb < KB; ++kb) {
+    for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
       for (int e = 0; e < 16; ++e) sacc[kb][e] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const s16x8 kf = *(const s16x8*)(ks_lds + kb * 32 * ROWB + koff[ks]);
-        sacc[kb] = E::mma(kf, qf[ks], sacc[kb]);
-      }
-    }
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) sacc[kb] = E::mma(kf[ks][kb], qf[ks], sacc[kb]);
 
     // diagonal chunk pair: key visible iff key_local <= query_local
     if (diag && (t + 1) * BN - 1 > qt * kBlockM) {
@@ -227,7 +225,7 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
         }
     }
 
-    // online softmax (csrc/ring_attention.cu:194-245); this lane's query is n
+    // this lane's query is n: in-register max, one exchange with the other half
     float mx = sacc[0][0];
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
@@ -247,7 +245,6 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
 
     // P^T = exp2(S^T k2 - m k2); row sum from the unrounded values (:242), operands
     // rounded to the storage type (:604)
-    s16x8 pf[KB][2];
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -261,9 +258,11 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
         }
         pf[kb][t2] = __builtin_bit_cast(s16x8, pv);
       }
-
-    // O^T += V^T P^T (csrc/ring_attention.cu:609).  MFMA slice (kb, t2) contracts over
-    // keys 32 kb + 16 t2 + {4 h + 0..3, 8 + 4 h + 0..3}, the keys this lane's P values belong to.
+  };
+  // O^T += V^T P^T (csrc/ring_attention.cu:609).  MFMA slice (kb, t2) contracts over keys
+  // 32 kb + 16 t2 + {4 h + 0..3, 8 + 4 h + 0..3}, the keys this lane's P values belong to.
+  auto pv_product = [&](int buf) {
+    const unsigned char* vs_lds = smem + (2 + buf) * TILE;
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -277,6 +276,27 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
           oacc[db] = E::mma(vf, pf[kb][t2], oacc[db]);
         }
       }
+  };
+
+  // Retire the Q loads here, with a wait the compiler can see: otherwise it places
+  // counted vmcnt waits at their first use inside the loop, and those would also
+  // drain the direct-to-LDS prefetch it does not know about.
+  __builtin_amdgcn_s_waitcnt(0);
+
+  // one barrier per tile at the top; K and V of tile t+1 are in flight while tile t is computed
+  issue_k(0, 0);
+  issue_v(0, 0);
+  for (int t = 0; t < n_tiles; ++t) {
+    const int buf = t & 1;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // tile t is in LDS; every wave is done with tile t-1
+    if (t + 1 < n_tiles) {
+      issue_k(t + 1, buf ^ 1);
+      issue_v(t + 1, buf ^ 1);
+    }
+    load_k_frags(buf);
+    scores_and_softmax(t);
+    pv_product(buf);
   }
 
   // epilogue (csrc/ring_attention.cu:621-633): normalise, emit partial O and LSE
