@@ -27,6 +27,8 @@
 //       ring steps (:439-443,597).  The merge is the algebraic equivalent on
 //       (O, LSE) pairs.
 #include "ringattn_kernels.h"
+#include <cstdlib>
+#include <type_traits>
 
 namespace ringattn {
 
@@ -319,6 +321,287 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   }
 }
 
+// ---- software-pipelined block kernel ---------------------------------------------------
+// Same math and data layout as block_attention_kernel, different schedule.  The KV chunk is
+// consumed in 32-key tiles held in two 4-deep LDS rings (K and V).  Block u of the loop
+// runs, in ONE instruction stream,
+//     MFMAs of S^T(u+1) = K(u+1) Q^T      next to   the exponentials of tile u,
+//     MFMAs of O^T += V(u)^T P(u)^T       next to   the row-max reduction of tile u+1,
+// so every wave feeds the matrix pipe and the VALU at the same time instead of alternating
+// between them.  The exponent offset m is a REFERENCE max: it is moved (with the rescale of
+// l and acc-O of csrc/ring_attention.cu:226-232) only when some row's tile max exceeds it by
+// more than 2^kLazyLog2, decided at the end of a block, which keeps the blocks free of
+// branches.  Until then p = exp2((s - m) k2) may exceed 1; O = acc / l and
+// LSE = (m k2 + log2 l) ln 2 do not depend on the choice of m.
+template <int DT, int D, int SCHED>
+__global__ __launch_bounds__(256, 2) void block_attention_pipe_kernel(const BlockStepArgs a) {
+  using E = Elem<DT>;
+  constexpr int BM = 128;          // query rows per workgroup (4 waves x 32)
+  constexpr int BN = 32;           // keys per tile
+  constexpr int NBUF = 4;          // ring depth of the K and of the V tiles
+  constexpr int CPR = D / 8;       // 16-byte chunks per row
+  constexpr int ROWB = D * 2;      // bytes per row
+  constexpr int TILE = BN * ROWB;  // bytes per tile
+  constexpr int KS = D / 16;       // contraction slices of QK^T
+  constexpr int DB = D / 32;       // 32-wide blocks of the head dim in PV
+  constexpr int LD = (BN * CPR) / 256;  // LDS-DMA instructions per wave per tile
+  constexpr float kLazyLog2 = 8.f;
+  static_assert(LD >= 1, "tile must split over 4 waves");
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * NBUF * TILE];  // K ring, V ring
+
+  const unsigned smem_base = lds_offset(smem);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 31, h = lane >> 5;
+
+  // workgroup -> (head, rank, q tile), XCD-aware as in block_attention_kernel
+  const int q_tiles = a.chunk / BM;
+  const int groups = a.n_active * a.BH;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int group = (slot / q_tiles) * 8 + xcd;
+  if (group >= groups) return;
+  const int ridx = group % a.n_active, bh = group / a.n_active;
+  const int r = a.rank_base + ridx;
+  int j = r + a.step;
+  if (j >= a.P) j -= a.P;
+  if (a.causal && j > r) return;
+  const bool diag = a.causal && (j == r);
+  int qt = slot % q_tiles;
+  if (diag) qt = q_tiles - 1 - qt;
+  const int n_tiles = diag ? ((qt + 1) * BM) / BN : a.chunk / BN;
+  const int first_masked = diag ? (qt * BM) / BN : n_tiles;  // tiles >= this need the causal mask
+
+  const int64_t head_off = (int64_t)bh * a.bh_stride;
+  const char* qbase = (const char*)a.q + (head_off + (int64_t)(r * a.chunk + qt * BM) * D) * 2;
+  const char* kbase = (const char*)a.k + (head_off + (int64_t)j * a.chunk * D) * 2;
+  const char* vbase = (const char*)a.v + (head_off + (int64_t)j * a.chunk * D) * 2;
+
+  s16x8 qf[KS];
+  {
+    const char* qrow = qbase + (int64_t)(32 * wave + n) * ROWB + h * 16;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const s16x8*)(qrow + ks * 32);
+  }
+  int goff_k[LD], goff_v[LD];
+#pragma unroll
+  for (int i = 0; i < LD; ++i) {
+    const int p = (wave * LD + i) * 64 + lane;
+    const int row = p / CPR, pc = p % CPR;
+    goff_k[i] = row * ROWB + ((pc ^ k_swizzle<D>(row)) << 4);
+    goff_v[i] = row * ROWB + ((pc ^ v_swizzle<D>(row)) << 4);
+  }
+  int koff[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) koff[ks] = n * ROWB + (((2 * ks + h) ^ k_swizzle<D>(n)) << 4);
+  int voff[DB];
+  {
+    const int s = lane & 15, g1 = (lane >> 4) & 1;
+    const int row8 = 4 * h + (s >> 2);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int c = 2 * (2 * db + g1) + ((s & 3) >> 1);
+      voff[db] = row8 * ROWB + ((c ^ v_swizzle<D>(row8)) << 4) + ((s & 1) << 3);
+    }
+  }
+
+  float m = -INFINITY;  // reference max (raw score units)
+  float ms = 0.f;       // m * k2, 0 while m is -inf (guard of csrc/ring_attention.cu:183)
+  float ls[4] = {0.f, 0.f, 0.f, 0.f};
+  f32x16 oacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
+  f32x16 s_even, s_odd;
+  s16x8 pf[2];
+
+  auto issue_k = [&](int t) {
+    const char* kt = kbase + (int64_t)t * TILE;
+    const unsigned kd = __builtin_amdgcn_readfirstlane(smem_base + (t & (NBUF - 1)) * TILE + wave * (LD * 1024));
+#pragma unroll
+    for (int i = 0; i < LD; ++i) load_lds_16(kt, goff_k[i], kd + i * 1024);
+  };
+  auto issue_v = [&](int t) {
+    const char* vt = vbase + (int64_t)t * TILE;
+    const unsigned vd = __builtin_amdgcn_readfirstlane(smem_base + (NBUF + (t & (NBUF - 1))) * TILE + wave * (LD * 1024));
+#pragma unroll
+    for (int i = 0; i < LD; ++i) load_lds_16(vt, goff_v[i], vd + i * 1024);
+  };
+  // S^T = K Q^T of one 32-key tile (csrc/ring_attention.cu:565)
+  auto qk = [&](f32x16& sacc, int kslot) {
+    const unsigned char* ks_lds = smem + kslot * TILE;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) sacc[e] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const s16x8 kfr = *(const s16x8*)(ks_lds + koff[ks]);
+      sacc = E::mma(kfr, qf[ks], sacc);
+    }
+  };
+  auto mask_tile = [&](f32x16& sacc, int t) {
+    if (t >= first_masked) {  // diagonal chunk pair: key visible iff key_local <= query_local
+      const int lim = qt * BM + 32 * wave + n - t * BN - 4 * h;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int key = 8 * (e >> 2) + (e & 3);
+        if (key > lim) sacc[e] = -INFINITY;
+      }
+    }
+  };
+  auto tile_max = [&](const f32x16& sacc) {
+    // two chains of max(max(m, a), b): the compiler folds each into one v_max3_f32
+    float m0 = sacc[0], m1 = sacc[1];
+#pragma unroll
+    for (int e = 2; e < 16; e += 4) {
+      m0 = fmaxf(fmaxf(m0, sacc[e]), sacc[e + 1]);
+      if (e + 3 < 16) m1 = fmaxf(fmaxf(m1, sacc[e + 2]), sacc[e + 3]);
+    }
+    return cross_half_max(fmaxf(m0, m1));
+  };
+  auto move_reference = [&](float tm) {
+    if (__builtin_amdgcn_ballot_w64((tm - m) * a.scale_log2 > kLazyLog2) != 0) {
+      const float cand = fmaxf(m, tm);
+      const float cs = (cand == -INFINITY) ? 0.f : cand * a.scale_log2;
+      const float alpha = __builtin_amdgcn_exp2f(m * a.scale_log2 - cs);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ls[i] *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
+      m = cand;
+      ms = cs;
+    }
+  };
+  // P^T = exp2(S^T k2 - m k2): row sum from the unrounded values (csrc/ring_attention.cu:242),
+  // MFMA operands rounded to the storage type (:604)
+  auto exponentials = [&](const f32x16& sacc) {
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      typename E::vec8 pv;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * t2 + e], a.scale_log2, -ms));
+        ls[e & 3] += p;
+        pv[e] = (typename E::type)p;
+      }
+      pf[t2] = __builtin_bit_cast(s16x8, pv);
+    }
+  };
+  // O^T += V^T P^T of one 32-key tile (csrc/ring_attention.cu:609)
+  auto pv_product = [&](int vslot) {
+    const unsigned char* vs_lds = smem + (NBUF + vslot) * TILE;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      const unsigned char* vrow = vs_lds + 16 * t2 * ROWB;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vrow + voff[db]));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vrow + 8 * ROWB + voff[db]));
+        const s16x8 vfr = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        oacc[db] = E::mma(vfr, pf[t2], oacc[db]);
+      }
+    }
+  };
+
+  // Block u.  Even blocks start with the barrier of the pair (u, u+1): K(u+1), K(u+2), V(u)
+  // and V(u+1), issued two blocks earlier, have landed, and every wave is past block u-1, so
+  // the ring slots of K(u-1), K(u), V(u-2), V(u-1) are free for K(u+3), K(u+4), V(u+2), V(u+3).
+  // STEADY blocks (all those tiles exist, tiles u+1 and u+2 unmasked) have compile-time ring
+  // slots and no conditions.
+  auto block = [&](auto slot_c, auto steady, int u) {
+    constexpr int SLOT = decltype(slot_c)::value;  // u mod 4 (STEADY) or u mod 2 (general)
+    constexpr bool STEADY = decltype(steady)::value;
+    f32x16& cur = (SLOT & 1) ? s_odd : s_even;
+    f32x16& nxt = (SLOT & 1) ? s_even : s_odd;
+    if (STEADY) {
+      if ((SLOT & 1) == 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        issue_k(u + 3);
+        issue_k(u + 4);
+        issue_v(u + 2);
+        issue_v(u + 3);
+      }
+      qk(nxt, (SLOT + 1) & 3);
+      exponentials(cur);
+      pv_product(SLOT);
+      const float tm = tile_max(nxt);
+      if constexpr (SCHED == 1) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+      }
+      move_reference(tm);
+    } else {
+      if ((u & 1) == 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (u + 3 < n_tiles) issue_k(u + 3);
+        if (u + 4 < n_tiles) issue_k(u + 4);
+        if (u + 2 < n_tiles) issue_v(u + 2);
+        if (u + 3 < n_tiles) issue_v(u + 3);
+      }
+      if (u + 1 < n_tiles) {
+        qk(nxt, (u + 1) & 3);
+        mask_tile(nxt, u + 1);
+      }
+      exponentials(cur);
+      pv_product(u & 3);
+      if (u + 1 < n_tiles) move_reference(tile_max(nxt));
+    }
+  };
+
+  __builtin_amdgcn_s_waitcnt(0);  // retire the Q loads with a wait the compiler can see
+  issue_k(0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (n_tiles > 1) issue_k(1);
+  if (n_tiles > 2) issue_k(2);
+  issue_v(0);
+  if (n_tiles > 1) issue_v(1);
+  qk(s_even, 0);
+  mask_tile(s_even, 0);
+  move_reference(tile_max(s_even));
+
+  using C0 = std::integral_constant<int, 0>;
+  using C1 = std::integral_constant<int, 1>;
+  using C2 = std::integral_constant<int, 2>;
+  using C3 = std::integral_constant<int, 3>;
+  // a steady pair (u, u+1), u even, needs u + 4 < n_tiles and u + 2 < first_masked
+  const int n_steady = min(n_tiles - 4, first_masked - 2);  // pairs starting at u < n_steady
+  int u = 0;
+  for (; u + 2 < n_steady; u += 4) {
+    block(C0{}, std::true_type{}, u);
+    block(C1{}, std::true_type{}, u + 1);
+    block(C2{}, std::true_type{}, u + 2);
+    block(C3{}, std::true_type{}, u + 3);
+  }
+  for (; u < n_tiles; ++u) {
+    if (u & 1) block(C1{}, std::false_type{}, u);
+    else block(C0{}, std::false_type{}, u);
+  }
+
+  // epilogue (csrc/ring_attention.cu:621-633): normalise, emit partial O and LSE
+  const float l = cross_half_sum((ls[0] + ls[1]) + (ls[2] + ls[3]));
+  const float inv = (l > 0.f) ? 1.f / l : 0.f;
+  const int row_g = r * a.chunk + qt * BM + 32 * wave + n;
+  float* orow = a.o_part + ((int64_t)bh * a.S + row_g) * D;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      f32x4 val;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) val[e] = oacc[db][4 * q4 + e] * inv;
+      *(f32x4*)(orow + 32 * db + 8 * q4 + 4 * h) = val;
+    }
+  if (h == 0) {
+    const float lse = (l > 0.f) ? (ms + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
+    a.lse_part[(int64_t)bh * a.S + row_g] = lse;
+  }
+}
+
 // ---- merge ------------------------------------------------------------------------
 template <int DT> struct Store8;
 template <> struct Store8<0> {
@@ -388,6 +671,18 @@ hipError_t launch_block_step(const BlockStepArgs& a, int dtype, int dim, hipStre
   const int q_tiles = a.chunk / kBlockM;
   const int groups = a.n_active * a.BH;
   const unsigned grid = (unsigned)(((groups + 7) / 8) * 8 * q_tiles);
+  static const int var = getenv("RINGATTN_VARIANT") ? atoi(getenv("RINGATTN_VARIANT")) : 0;
+#define RA_PIPE(SCHED)                                                                                  \
+  {                                                                                                     \
+    if (dtype == 0 && dim == 64) block_attention_pipe_kernel<0, 64, SCHED><<<grid, 256, 0, stream>>>(a);        \
+    else if (dtype == 0 && dim == 128) block_attention_pipe_kernel<0, 128, SCHED><<<grid, 256, 0, stream>>>(a); \
+    else if (dtype == 1 && dim == 64) block_attention_pipe_kernel<1, 64, SCHED><<<grid, 256, 0, stream>>>(a);   \
+    else if (dtype == 1 && dim == 128) block_attention_pipe_kernel<1, 128, SCHED><<<grid, 256, 0, stream>>>(a); \
+    else return hipErrorInvalidValue;                                                                   \
+    return hipGetLastError();                                                                           \
+  }
+  if (var == 1) RA_PIPE(0)
+  if (var == 2) RA_PIPE(1)
   if (dtype == 0 && dim == 64) block_attention_kernel<0, 64, 64><<<grid, 256, 0, stream>>>(a);
   else if (dtype == 0 && dim == 128) block_attention_kernel<0, 128, 64><<<grid, 256, 0, stream>>>(a);
   else if (dtype == 1 && dim == 64) block_attention_kernel<1, 64, 64><<<grid, 256, 0, stream>>>(a);
