@@ -123,6 +123,8 @@ def main():
         "traffic": MEASURED_TRAFFIC.get(w.name),
         "launches_per_step": w.npes, "avg_launch_ms": round(float(np.mean(block_ms)), 4),
         "avg_launch_flop": float(np.mean(launch_flops)),
+        "per_step_ms": [round(float(x), 4) for x in block_ms],
+        "per_step_tflops": [round(f / (t * 1e-3) / 1e12, 1) for f, t in zip(launch_flops, block_ms)],
     }
     # merge: algorithmic bytes = active parts * (4 d + 4) read + (2 d + 4) written, per row
     P = w.npes

@@ -17,17 +17,20 @@
 //           reductions plus one cross-half exchange, and the probabilities are
 //           already in B-operand layout for O^T += V^T P^T -- the MFMA analogue
 //           of convert_layout_rowcol_Aregs (:260-276);
-//         * K and V tiles go HBM -> LDS directly (global_load_lds_dwordx4),
-//           double-buffered, one barrier per tile; bank conflicts are removed
-//           by an XOR swizzle applied on the global-address side;
+//         * K and V go HBM -> LDS directly (global_load_lds_dwordx4) in 32-key
+//           tiles, through two 4-deep rings, one barrier per two tiles; bank
+//           conflicts are removed by an XOR swizzle applied on the
+//           global-address side;
 //         * V^T operands come from ds_read_b64_tr_b16 (the LDS transpose read),
-//           replacing ldmatrix.trans of csrc/kernel_traits.h:39.
+//           replacing ldmatrix.trans of csrc/kernel_traits.h:39;
+//         * the loop is software-pipelined: the MFMAs of tile u+1's scores run
+//           next to the exponentials of tile u (see the kernel's comment).
 //   merge_kernel : P-way merge of the per-step (O, LSE) partials.  The reference
 //       has no such function: it carries (max, sum, acc-O) in registers across
 //       ring steps (:439-443,597).  The merge is the algebraic equivalent on
 //       (O, LSE) pairs.
 #include "ringattn_kernels.h"
-#include <cstdlib>
+
 #include <type_traits>
 
 namespace ringattn {
@@ -77,9 +80,9 @@ static __device__ __forceinline__ void swap_halves(float& a, float& b) {
   asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
 }
 static __device__ __forceinline__ float cross_half_max(float x) {
-  float a = x, b = x;
-  swap_halves(a, b);
-  return fmaxf(a, b);
+  float a = x, b = x, r;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %1, %2\n\ts_nop 1\n\tv_max_f32 %0, %1, %2" : "=v"(r), "+v"(a), "+v"(b));
+  return r;
 }
 static __device__ __forceinline__ float cross_half_sum(float x) {
   float a = x, b = x;
@@ -98,245 +101,24 @@ template <int D> static __device__ __forceinline__ int v_swizzle(int row) {
                   : ((((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1));
 }
 
-template <int DT, int D, int BN>
-__global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStepArgs a) {
-  using E = Elem<DT>;
-  constexpr int CPR = D / 8;       // 16-byte chunks per row
-  constexpr int ROWB = D * 2;      // bytes per row
-  constexpr int TILE = BN * ROWB;  // bytes per K or V tile
-  constexpr int KB = BN / 32;      // 32-key blocks per tile
-  constexpr int KS = D / 16;       // contraction slices of QK^T
-  constexpr int DB = D / 32;       // 32-wide blocks of the head dim in PV
-  constexpr int LD_PER_WAVE = (BN * CPR) / 256;  // LDS-DMA instructions per wave per tile
-  static_assert(LD_PER_WAVE >= 1 && (BN * CPR) % 256 == 0, "tile must split over 4 waves");
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[4 * TILE];  // K0 K1 V0 V1
-
-  const unsigned smem_base = lds_offset(smem);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n = lane & 31, h = lane >> 5;
-
-  // workgroup -> (head, rank, q tile).  Consecutive workgroup ids go round-robin over
-  // the 8 XCDs, so all q tiles of one (head, rank) -- which stream the same KV chunk --
-  // are placed on one XCD and share its L2.
-  const int q_tiles = a.chunk / kBlockM;
-  const int groups = a.n_active * a.BH;
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int group = (slot / q_tiles) * 8 + xcd;
-  if (group >= groups) return;
-  const int ridx = group % a.n_active, bh = group / a.n_active;
-  const int r = a.rank_base + ridx;
-  int j = r + a.step;
-  if (j >= a.P) j -= a.P;
-  if (a.causal && j > r) return;  // fully masked pair: never launched by the host loop
-  const bool diag = a.causal && (j == r);
-  int qt = slot % q_tiles;
-  if (diag) qt = q_tiles - 1 - qt;  // heaviest q tiles first
-  const int n_tiles = diag ? ((qt + 1) * kBlockM) / BN : a.chunk / BN;
-
-  const int64_t head_off = (int64_t)bh * a.bh_stride;
-  const char* qbase = (const char*)a.q + (head_off + (int64_t)(r * a.chunk + qt * kBlockM) * D) * 2;
-  const char* kbase = (const char*)a.k + (head_off + (int64_t)j * a.chunk * D) * 2;
-  const char* vbase = (const char*)a.v + (head_off + (int64_t)j * a.chunk * D) * 2;
-
-  // Q fragment: B operand of S^T = K Q^T.  Lane (n, h) holds Q[row n][16 ks + 8 h .. +8).
-  s16x8 qf[KS];
-  {
-    const char* qrow = qbase + (int64_t)(32 * wave + n) * ROWB + h * 16;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const s16x8*)(qrow + ks * 32);
-  }
-
-  // per-lane source offsets of the direct-to-LDS tile loads (swizzle on the global side)
-  int goff_k[LD_PER_WAVE], goff_v[LD_PER_WAVE];
-#pragma unroll
-  for (int i = 0; i < LD_PER_WAVE; ++i) {
-    const int p = (wave * LD_PER_WAVE + i) * 64 + lane;
-    const int row = p / CPR, pc = p % CPR;
-    goff_k[i] = row * ROWB + ((pc ^ k_swizzle<D>(row)) << 4);
-    goff_v[i] = row * ROWB + ((pc ^ v_swizzle<D>(row)) << 4);
-  }
-  // K operand read offsets: lane (n, h) reads row 32 kb + n, logical chunk 2 ks + h
-  int koff[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) koff[ks] = n * ROWB + (((2 * ks + h) ^ k_swizzle<D>(n)) << 4);
-  // V^T operand read offsets (ds_read_b64_tr_b16): within a group of 16 lanes, lane s
-  // points at V[k0 + s/4][dbase + 4 (s%4) .. +4) and receives V[k0 .. k0+4)[dbase + s].
-  int voff[DB];
-  {
-    const int s = lane & 15, g1 = (lane >> 4) & 1;
-    const int row8 = 4 * h + (s >> 2);
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const int c = 2 * (2 * db + g1) + ((s & 3) >> 1);
-      voff[db] = row8 * ROWB + ((c ^ v_swizzle<D>(row8)) << 4) + ((s & 1) << 3);
-    }
-  }
-
-  float m = -INFINITY, lsum = 0.f;
-  f32x16 oacc[DB];
-#pragma unroll
-  for (int db = 0; db < DB; ++db)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
-
-  // direct-to-LDS loads of one K or V tile (this wave's share)
-  auto issue_k = [&](int t, int buf) {
-    const char* kt = kbase + (int64_t)t * TILE;
-    const unsigned kd = __builtin_amdgcn_readfirstlane(smem_base + buf * TILE + wave * (LD_PER_WAVE * 1024));
-#pragma unroll
-    for (int i = 0; i < LD_PER_WAVE; ++i) load_lds_16(kt, goff_k[i], kd + i * 1024);
-  };
-  auto issue_v = [&](int t, int buf) {
-    const char* vt = vbase + (int64_t)t * TILE;
-    const unsigned vd = __builtin_amdgcn_readfirstlane(smem_base + (2 + buf) * TILE + wave * (LD_PER_WAVE * 1024));
-#pragma unroll
-    for (int i = 0; i < LD_PER_WAVE; ++i) load_lds_16(vt, goff_v[i], vd + i * 1024);
-  };
-  // K fragments (A operand of S^T = K Q^T) of a whole tile, LDS -> registers
-  s16x8 kf[KS][KB];
-  auto load_k_frags = [&](int buf) {
-    const unsigned char* ks_lds = smem + buf * TILE;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb) kf[ks][kb] = *(const s16x8*)(ks_lds + kb * 32 * ROWB + koff[ks]);
-  };
-  // S^T = K Q^T : keys x queries, fp32 accumulate (csrc/ring_attention.cu:565), then the
-  // online softmax (:194-245).  Leaves P^T, rounded to the storage type, in pf as B operands.
-  s16x8 pf[KB][2];
-  auto scores_and_softmax = [&](int t) {
-    f32x16 sacc[KB];
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) sacc[kb][e] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb) sacc[kb] = E::mma(kf[ks][kb], qf[ks], sacc[kb]);
-
-    // diagonal chunk pair: key visible iff key_local <= query_local
-    if (diag && (t + 1) * BN - 1 > qt * kBlockM) {
-      const int lim = qt * kBlockM + 32 * wave + n - t * BN - 4 * h;
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int key = 32 * kb + 8 * (e >> 2) + (e & 3);
-          if (key > lim) sacc[kb][e] = -INFINITY;
-        }
-    }
-
-    // this lane's query is n: in-register max, one exchange with the other half
-    float mx = sacc[0][0];
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[kb][e]);
-    mx = cross_half_max(mx);
-    const float m_new = fmaxf(m, mx);
-    // all-masked guard of scale_apply_exp2 (csrc/ring_attention.cu:183)
-    const float ms = (m_new == -INFINITY) ? 0.f : m_new * a.scale_log2;
-    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {  // some row's running max moved
-      const float alpha = __builtin_amdgcn_exp2f(m * a.scale_log2 - ms);
-      lsum *= alpha;
-#pragma unroll
-      for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
-    }
-    m = m_new;
-
-    // P^T = exp2(S^T k2 - m k2); row sum from the unrounded values (:242), operands
-    // rounded to the storage type (:604)
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2) {
-        typename E::vec8 pv;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][8 * t2 + e], a.scale_log2, -ms));
-          lsum += p;
-          pv[e] = (typename E::type)p;
-        }
-        pf[kb][t2] = __builtin_bit_cast(s16x8, pv);
-      }
-  };
-  // O^T += V^T P^T (csrc/ring_attention.cu:609).  MFMA slice (kb, t2) contracts over keys
-  // 32 kb + 16 t2 + {4 h + 0..3, 8 + 4 h + 0..3}, the keys this lane's P values belong to.
-  auto pv_product = [&](int buf) {
-    const unsigned char* vs_lds = smem + (2 + buf) * TILE;
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2) {
-        const unsigned char* vrow = vs_lds + (32 * kb + 16 * t2) * ROWB;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vrow + voff[db]));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vrow + 8 * ROWB + voff[db]));
-          const s16x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          oacc[db] = E::mma(vf, pf[kb][t2], oacc[db]);
-        }
-      }
-  };
-
-  // Retire the Q loads here, with a wait the compiler can see: otherwise it places
-  // counted vmcnt waits at their first use inside the loop, and those would also
-  // drain the direct-to-LDS prefetch it does not know about.
-  __builtin_amdgcn_s_waitcnt(0);
-
-  // one barrier per tile at the top; K and V of tile t+1 are in flight while tile t is computed
-  issue_k(0, 0);
-  issue_v(0, 0);
-  for (int t = 0; t < n_tiles; ++t) {
-    const int buf = t & 1;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();  // tile t is in LDS; every wave is done with tile t-1
-    if (t + 1 < n_tiles) {
-      issue_k(t + 1, buf ^ 1);
-      issue_v(t + 1, buf ^ 1);
-    }
-    load_k_frags(buf);
-    scores_and_softmax(t);
-    pv_product(buf);
-  }
-
-  // epilogue (csrc/ring_attention.cu:621-633): normalise, emit partial O and LSE
-  const float l = cross_half_sum(lsum);
-  const float inv = (l > 0.f) ? 1.f / l : 0.f;
-  const int row_g = r * a.chunk + qt * kBlockM + 32 * wave + n;
-  float* orow = a.o_part + ((int64_t)bh * a.S + row_g) * D;
-#pragma unroll
-  for (int db = 0; db < DB; ++db)
-#pragma unroll
-    for (int q4 = 0; q4 < 4; ++q4) {
-      f32x4 val;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) val[e] = oacc[db][4 * q4 + e] * inv;
-      *(f32x4*)(orow + 32 * db + 8 * q4 + 4 * h) = val;
-    }
-  if (h == 0) {
-    const float lse = (l > 0.f) ? (m * a.scale_log2 + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
-    a.lse_part[(int64_t)bh * a.S + row_g] = lse;
-  }
-}
-
-// ---- software-pipelined block kernel ---------------------------------------------------
-// Same math and data layout as block_attention_kernel, different schedule.  The KV chunk is
-// consumed in 32-key tiles held in two 4-deep LDS rings (K and V).  Block u of the loop
-// runs, in ONE instruction stream,
+// ---- block attention: one ring step for every active virtual rank ------------------------
+// The KV chunk is consumed in 32-key tiles held in two 4-deep LDS rings (K and V), filled by
+// direct-to-LDS loads that run two blocks ahead.  Block u of the loop runs, in ONE
+// instruction stream,
 //     MFMAs of S^T(u+1) = K(u+1) Q^T      next to   the exponentials of tile u,
 //     MFMAs of O^T += V(u)^T P(u)^T       next to   the row-max reduction of tile u+1,
 // so every wave feeds the matrix pipe and the VALU at the same time instead of alternating
 // between them.  The exponent offset m is a REFERENCE max: it is moved (with the rescale of
 // l and acc-O of csrc/ring_attention.cu:226-232) only when some row's tile max exceeds it by
 // more than 2^kLazyLog2, decided at the end of a block, which keeps the blocks free of
-// branches.  Until then p = exp2((s - m) k2) may exceed 1; O = acc / l and
-// LSE = (m k2 + log2 l) ln 2 do not depend on the choice of m.
-template <int DT, int D, int SCHED>
-__global__ __launch_bounds__(256, 2) void block_attention_pipe_kernel(const BlockStepArgs a) {
+// branches.  Until then p = exp2((s - m) k2) may exceed 1 (by at most 2^kLazyLog2, well
+// inside fp16 and bf16 range); O = acc / l and LSE = (m k2 + log2 l) ln 2 do not depend on
+// the choice of m.
+template <int DT, int D>
+__global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStepArgs a) {
   using E = Elem<DT>;
-  constexpr int BM = 128;          // query rows per workgroup (4 waves x 32)
+  constexpr int QB = 1;            // 32-query blocks per wave
+  constexpr int BM = kBlockM;      // query rows per workgroup: 4 waves x 32
   constexpr int BN = 32;           // keys per tile
   constexpr int NBUF = 4;          // ring depth of the K and of the V tiles
   constexpr int CPR = D / 8;       // 16-byte chunks per row
@@ -375,11 +157,13 @@ __global__ __launch_bounds__(256, 2) void block_attention_pipe_kernel(const Bloc
   const char* kbase = (const char*)a.k + (head_off + (int64_t)j * a.chunk * D) * 2;
   const char* vbase = (const char*)a.v + (head_off + (int64_t)j * a.chunk * D) * 2;
 
-  s16x8 qf[KS];
-  {
-    const char* qrow = qbase + (int64_t)(32 * wave + n) * ROWB + h * 16;
+  // this lane's query rows (local to the q tile): 32 QB wave + 32 qb + n
+  s16x8 qf[QB][KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const s16x8*)(qrow + ks * 32);
+  for (int qb = 0; qb < QB; ++qb) {
+    const char* qrow = qbase + (int64_t)(32 * QB * wave + 32 * qb + n) * ROWB + h * 16;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[qb][ks] = *(const s16x8*)(qrow + ks * 32);
   }
   int goff_k[LD], goff_v[LD];
 #pragma unroll
@@ -403,16 +187,23 @@ __global__ __launch_bounds__(256, 2) void block_attention_pipe_kernel(const Bloc
     }
   }
 
-  float m = -INFINITY;  // reference max (raw score units)
-  float ms = 0.f;       // m * k2, 0 while m is -inf (guard of csrc/ring_attention.cu:183)
-  float ls[4] = {0.f, 0.f, 0.f, 0.f};
-  f32x16 oacc[DB];
+  float m[QB];   // reference max per query block (raw score units)
+  float ms[QB];  // m * k2, 0 while m is -inf (guard of csrc/ring_attention.cu:183)
+  float ls[QB][4];
+  f32x16 oacc[QB][DB];
 #pragma unroll
-  for (int db = 0; db < DB; ++db)
+  for (int qb = 0; qb < QB; ++qb) {
+    m[qb] = -INFINITY;
+    ms[qb] = 0.f;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
-  f32x16 s_even, s_odd;
-  s16x8 pf[2];
+    for (int i = 0; i < 4; ++i) ls[qb][i] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) oacc[qb][db][e] = 0.f;
+  }
+  f32x16 s_even[QB], s_odd[QB];
+  s16x8 pf[QB][2];
 
   auto issue_k = [&](int t) {
     const char* kt = kbase + (int64_t)t * TILE;
@@ -426,66 +217,84 @@ __global__ __launch_bounds__(256, 2) void block_attention_pipe_kernel(const Bloc
 #pragma unroll
     for (int i = 0; i < LD; ++i) load_lds_16(vt, goff_v[i], vd + i * 1024);
   };
-  // S^T = K Q^T of one 32-key tile (csrc/ring_attention.cu:565)
-  auto qk = [&](f32x16& sacc, int kslot) {
+  // S^T = K Q^T of one 32-key tile (csrc/ring_attention.cu:565); each K fragment feeds all
+  // QB query blocks of the wave
+  auto qk = [&](f32x16(&sacc)[QB], int kslot) {
     const unsigned char* ks_lds = smem + kslot * TILE;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) sacc[e] = 0.f;
+    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) sacc[qb][e] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const s16x8 kfr = *(const s16x8*)(ks_lds + koff[ks]);
-      sacc = E::mma(kfr, qf[ks], sacc);
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) sacc[qb] = E::mma(kfr, qf[qb][ks], sacc[qb]);
     }
   };
-  auto mask_tile = [&](f32x16& sacc, int t) {
+  auto mask_tile = [&](f32x16(&sacc)[QB], int t) {
     if (t >= first_masked) {  // diagonal chunk pair: key visible iff key_local <= query_local
-      const int lim = qt * BM + 32 * wave + n - t * BN - 4 * h;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int key = 8 * (e >> 2) + (e & 3);
-        if (key > lim) sacc[e] = -INFINITY;
+      for (int qb = 0; qb < QB; ++qb) {
+        const int lim = qt * BM + 32 * QB * wave + 32 * qb + n - t * BN - 4 * h;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int key = 8 * (e >> 2) + (e & 3);
+          if (key > lim) sacc[qb][e] = -INFINITY;
+        }
       }
     }
   };
-  auto tile_max = [&](const f32x16& sacc) {
-    // two chains of max(max(m, a), b): the compiler folds each into one v_max3_f32
-    float m0 = sacc[0], m1 = sacc[1];
+  // max(m, row max of the tile): two chains of max(max(x, a), b) seeded with the reference
+  // max, each link one v_max3_f32; one exchange between the halves of the wave
+  auto tile_max = [&](const f32x16& sacc, float mref) {
+    float m0 = mref, m1 = mref;
 #pragma unroll
-    for (int e = 2; e < 16; e += 4) {
+    for (int e = 0; e < 16; e += 4) {
       m0 = fmaxf(fmaxf(m0, sacc[e]), sacc[e + 1]);
-      if (e + 3 < 16) m1 = fmaxf(fmaxf(m1, sacc[e + 2]), sacc[e + 3]);
+      m1 = fmaxf(fmaxf(m1, sacc[e + 2]), sacc[e + 3]);
     }
     return cross_half_max(fmaxf(m0, m1));
   };
-  auto move_reference = [&](float tm) {
-    if (__builtin_amdgcn_ballot_w64((tm - m) * a.scale_log2 > kLazyLog2) != 0) {
-      const float cand = fmaxf(m, tm);
-      const float cs = (cand == -INFINITY) ? 0.f : cand * a.scale_log2;
-      const float alpha = __builtin_amdgcn_exp2f(m * a.scale_log2 - cs);
+  // cand = max(m, tile max).  The reference moves when some row's cand is far above it (or it
+  // is still unset): rescale of l and acc-O as in csrc/ring_attention.cu:226-232.
+  auto move_reference = [&](const float (&cand)[QB]) {
+    bool far = false;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) ls[i] *= alpha;
+    for (int qb = 0; qb < QB; ++qb) far = far || ((cand[qb] - m[qb]) * a.scale_log2 > kLazyLog2);
+    if (__builtin_amdgcn_ballot_w64(far) != 0) {
 #pragma unroll
-      for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
-      m = cand;
-      ms = cs;
+      for (int qb = 0; qb < QB; ++qb) {
+        const float cs = (cand[qb] == -INFINITY) ? 0.f : cand[qb] * a.scale_log2;
+        const float alpha = __builtin_amdgcn_exp2f(m[qb] * a.scale_log2 - cs);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ls[qb][i] *= alpha;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) oacc[qb][db] *= alpha;
+        m[qb] = cand[qb];
+        ms[qb] = cs;
+      }
     }
   };
   // P^T = exp2(S^T k2 - m k2): row sum from the unrounded values (csrc/ring_attention.cu:242),
   // MFMA operands rounded to the storage type (:604)
-  auto exponentials = [&](const f32x16& sacc) {
+  auto exponentials = [&](const f32x16(&sacc)[QB]) {
 #pragma unroll
-    for (int t2 = 0; t2 < 2; ++t2) {
-      typename E::vec8 pv;
+    for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * t2 + e], a.scale_log2, -ms));
-        ls[e & 3] += p;
-        pv[e] = (typename E::type)p;
+      for (int t2 = 0; t2 < 2; ++t2) {
+        typename E::vec8 pv;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qb][8 * t2 + e], a.scale_log2, -ms[qb]));
+          ls[qb][e & 3] += p;
+          pv[e] = (typename E::type)p;
+        }
+        pf[qb][t2] = __builtin_bit_cast(s16x8, pv);
       }
-      pf[t2] = __builtin_bit_cast(s16x8, pv);
-    }
   };
-  // O^T += V^T P^T of one 32-key tile (csrc/ring_attention.cu:609)
+  // O^T += V^T P^T of one 32-key tile (csrc/ring_attention.cu:609); each V^T fragment feeds
+  // all QB query blocks of the wave
   auto pv_product = [&](int vslot) {
     const unsigned char* vs_lds = smem + (NBUF + vslot) * TILE;
 #pragma unroll
@@ -496,9 +305,14 @@ __global__ __launch_bounds__(256, 2) void block_attention_pipe_kernel(const Bloc
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vrow + voff[db]));
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vrow + 8 * ROWB + voff[db]));
         const s16x8 vfr = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        oacc[db] = E::mma(vfr, pf[t2], oacc[db]);
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) oacc[qb][db] = E::mma(vfr, pf[qb][t2], oacc[qb][db]);
       }
     }
+  };
+  auto tile_maxes = [&](const f32x16(&sacc)[QB], float (&cand)[QB]) {
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) cand[qb] = tile_max(sacc[qb], m[qb]);
   };
 
   // Block u.  Even blocks start with the barrier of the pair (u, u+1): K(u+1), K(u+2), V(u)
@@ -509,8 +323,9 @@ __global__ __launch_bounds__(256, 2) void block_attention_pipe_kernel(const Bloc
   auto block = [&](auto slot_c, auto steady, int u) {
     constexpr int SLOT = decltype(slot_c)::value;  // u mod 4 (STEADY) or u mod 2 (general)
     constexpr bool STEADY = decltype(steady)::value;
-    f32x16& cur = (SLOT & 1) ? s_odd : s_even;
-    f32x16& nxt = (SLOT & 1) ? s_even : s_odd;
+    f32x16(&cur)[QB] = (SLOT & 1) ? s_odd : s_even;
+    f32x16(&nxt)[QB] = (SLOT & 1) ? s_even : s_odd;
+    float cand[QB];
     if (STEADY) {
       if ((SLOT & 1) == 0) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -523,16 +338,16 @@ __global__ __launch_bounds__(256, 2) void block_attention_pipe_kernel(const Bloc
       qk(nxt, (SLOT + 1) & 3);
       exponentials(cur);
       pv_product(SLOT);
-      const float tm = tile_max(nxt);
-      if constexpr (SCHED == 1) {
+      tile_maxes(nxt, cand);
+      // scheduling hint: in the first half of the block every MFMA is preceded by one and
+      // followed by two LDS reads, so the reads run ahead of the MFMAs that consume them
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        }
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
       }
-      move_reference(tm);
+      move_reference(cand);
     } else {
       if ((u & 1) == 0) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -548,7 +363,10 @@ __global__ __launch_bounds__(256, 2) void block_attention_pipe_kernel(const Bloc
       }
       exponentials(cur);
       pv_product(u & 3);
-      if (u + 1 < n_tiles) move_reference(tile_max(nxt));
+      if (u + 1 < n_tiles) {
+        tile_maxes(nxt, cand);
+        move_reference(cand);
+      }
     }
   };
 
@@ -560,9 +378,13 @@ __global__ __launch_bounds__(256, 2) void block_attention_pipe_kernel(const Bloc
   if (n_tiles > 2) issue_k(2);
   issue_v(0);
   if (n_tiles > 1) issue_v(1);
-  qk(s_even, 0);
-  mask_tile(s_even, 0);
-  move_reference(tile_max(s_even));
+  {
+    float cand[QB];
+    qk(s_even, 0);
+    mask_tile(s_even, 0);
+    tile_maxes(s_even, cand);
+    move_reference(cand);
+  }
 
   using C0 = std::integral_constant<int, 0>;
   using C1 = std::integral_constant<int, 1>;
@@ -583,22 +405,25 @@ __global__ __launch_bounds__(256, 2) void block_attention_pipe_kernel(const Bloc
   }
 
   // epilogue (csrc/ring_attention.cu:621-633): normalise, emit partial O and LSE
-  const float l = cross_half_sum((ls[0] + ls[1]) + (ls[2] + ls[3]));
-  const float inv = (l > 0.f) ? 1.f / l : 0.f;
-  const int row_g = r * a.chunk + qt * BM + 32 * wave + n;
-  float* orow = a.o_part + ((int64_t)bh * a.S + row_g) * D;
 #pragma unroll
-  for (int db = 0; db < DB; ++db)
+  for (int qb = 0; qb < QB; ++qb) {
+    const float l = cross_half_sum((ls[qb][0] + ls[qb][1]) + (ls[qb][2] + ls[qb][3]));
+    const float inv = (l > 0.f) ? 1.f / l : 0.f;
+    const int row_g = r * a.chunk + qt * BM + 32 * QB * wave + 32 * qb + n;
+    float* orow = a.o_part + ((int64_t)bh * a.S + row_g) * D;
 #pragma unroll
-    for (int q4 = 0; q4 < 4; ++q4) {
-      f32x4 val;
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) val[e] = oacc[db][4 * q4 + e] * inv;
-      *(f32x4*)(orow + 32 * db + 8 * q4 + 4 * h) = val;
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 val;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) val[e] = oacc[qb][db][4 * q4 + e] * inv;
+        *(f32x4*)(orow + 32 * db + 8 * q4 + 4 * h) = val;
+      }
+    if (h == 0) {
+      const float lse = (l > 0.f) ? (ms[qb] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
+      a.lse_part[(int64_t)bh * a.S + row_g] = lse;
     }
-  if (h == 0) {
-    const float lse = (l > 0.f) ? (ms + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
-    a.lse_part[(int64_t)bh * a.S + row_g] = lse;
   }
 }
 
@@ -671,22 +496,10 @@ hipError_t launch_block_step(const BlockStepArgs& a, int dtype, int dim, hipStre
   const int q_tiles = a.chunk / kBlockM;
   const int groups = a.n_active * a.BH;
   const unsigned grid = (unsigned)(((groups + 7) / 8) * 8 * q_tiles);
-  static const int var = getenv("RINGATTN_VARIANT") ? atoi(getenv("RINGATTN_VARIANT")) : 0;
-#define RA_PIPE(SCHED)                                                                                  \
-  {                                                                                                     \
-    if (dtype == 0 && dim == 64) block_attention_pipe_kernel<0, 64, SCHED><<<grid, 256, 0, stream>>>(a);        \
-    else if (dtype == 0 && dim == 128) block_attention_pipe_kernel<0, 128, SCHED><<<grid, 256, 0, stream>>>(a); \
-    else if (dtype == 1 && dim == 64) block_attention_pipe_kernel<1, 64, SCHED><<<grid, 256, 0, stream>>>(a);   \
-    else if (dtype == 1 && dim == 128) block_attention_pipe_kernel<1, 128, SCHED><<<grid, 256, 0, stream>>>(a); \
-    else return hipErrorInvalidValue;                                                                   \
-    return hipGetLastError();                                                                           \
-  }
-  if (var == 1) RA_PIPE(0)
-  if (var == 2) RA_PIPE(1)
-  if (dtype == 0 && dim == 64) block_attention_kernel<0, 64, 64><<<grid, 256, 0, stream>>>(a);
-  else if (dtype == 0 && dim == 128) block_attention_kernel<0, 128, 64><<<grid, 256, 0, stream>>>(a);
-  else if (dtype == 1 && dim == 64) block_attention_kernel<1, 64, 64><<<grid, 256, 0, stream>>>(a);
-  else if (dtype == 1 && dim == 128) block_attention_kernel<1, 128, 64><<<grid, 256, 0, stream>>>(a);
+  if (dtype == 0 && dim == 64) block_attention_kernel<0, 64><<<grid, 256, 0, stream>>>(a);
+  else if (dtype == 0 && dim == 128) block_attention_kernel<0, 128><<<grid, 256, 0, stream>>>(a);
+  else if (dtype == 1 && dim == 64) block_attention_kernel<1, 64><<<grid, 256, 0, stream>>>(a);
+  else if (dtype == 1 && dim == 128) block_attention_kernel<1, 128><<<grid, 256, 0, stream>>>(a);
   else return hipErrorInvalidValue;
   return hipGetLastError();
 }
