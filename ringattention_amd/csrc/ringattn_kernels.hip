@@ -46,9 +46,11 @@ typedef short s16x8 __attribute__((ext_vector_type(8)));
 // at lds_addr + 16 i (lds_addr is wave-uniform and travels in M0).  Written as inline
 // asm so the compiler does not serialise later LDS reads behind the transfer; the
 // kernel waits for it explicitly (s_waitcnt vmcnt(0)) before the tile barrier.
+// No "memory" clobber: a transfer only ever targets a ring slot that no LDS read between
+// the surrounding barriers touches, so the compiler may move LDS reads across it.
 // Nothing else in these kernels uses M0.
 static __device__ __forceinline__ void load_lds_16(const void* base, int voff, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base));
 }
 static __device__ __forceinline__ unsigned lds_offset(const void* p) {
   return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
@@ -316,8 +318,9 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   };
 
   // Block u.  Even blocks start with the barrier of the pair (u, u+1): K(u+1), K(u+2), V(u)
-  // and V(u+1), issued two blocks earlier, have landed, and every wave is past block u-1, so
-  // the ring slots of K(u-1), K(u), V(u-2), V(u-1) are free for K(u+3), K(u+4), V(u+2), V(u+3).
+  // and V(u+1), issued during the previous pair, have landed, and every wave is past block
+  // u-1, so the ring slots of K(u-1), K(u), V(u-2), V(u-1) are free for K(u+3), K(u+4),
+  // V(u+2), V(u+3), which are issued during this pair.
   // STEADY blocks (all those tiles exist, tiles u+1 and u+2 unmasked) have compile-time ring
   // slots and no conditions.
   auto block = [&](auto slot_c, auto steady, int u) {
@@ -327,16 +330,19 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
     f32x16(&nxt)[QB] = (SLOT & 1) ? s_even : s_odd;
     float cand[QB];
     if (STEADY) {
+      // the four tile loads of a pair are spread over its two blocks instead of being
+      // issued in one burst behind the barrier
       if ((SLOT & 1) == 0) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         issue_k(u + 3);
-        issue_k(u + 4);
-        issue_v(u + 2);
-        issue_v(u + 3);
+      } else {
+        issue_v(u + 1);
       }
       qk(nxt, (SLOT + 1) & 3);
       exponentials(cur);
+      if ((SLOT & 1) == 0) issue_k(u + 4);
+      else issue_v(u + 2);
       pv_product(SLOT);
       tile_maxes(nxt, cand);
       // scheduling hint: in the first half of the block every MFMA is preceded by one and
