@@ -459,29 +459,56 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
   const int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / TPR;
   if (row >= a.rows) return;
   const int c8 = threadIdx.x % TPR;
-  int first_wrapped = 1;  // parts s >= first_wrapped are active (besides s == 0)
+  // active parts of this row: part 0 and parts first_wrapped .. n_parts-1 (ring), or all
+  int first_wrapped = 1;
   if (a.causal_ring) {
     const int r = (int)((row % a.S) / a.chunk);
     first_wrapped = a.P - r;
   }
+  const int n_act = a.n_parts - first_wrapped + 1;
+  auto part_of = [&](int i) { return i == 0 ? 0 : first_wrapped + i - 1; };
+  const float* lse_row = a.lse_parts + row;
+  const float* o_row = a.o_parts + row * D + c8 * 8;
+  const int64_t lse_stride = a.part_stride_rows, o_stride = a.part_stride_rows * D;
+
   float mx = -INFINITY;
-  for (int s = 0; s < a.n_parts; ++s) {
-    if (s != 0 && s < first_wrapped) continue;
-    mx = fmaxf(mx, a.lse_parts[s * a.part_stride_rows + row]);
-  }
+  for (int i = 0; i < n_act; ++i) mx = fmaxf(mx, lse_row[part_of(i) * lse_stride]);
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   float wsum = 0.f;
   if (mx != -INFINITY) {
-    for (int s = 0; s < a.n_parts; ++s) {
-      if (s != 0 && s < first_wrapped) continue;
-      const float L = a.lse_parts[s * a.part_stride_rows + row];
-      if (L == -INFINITY) continue;  // identity element
-      const float w = __expf(L - mx);
+    // four parts per iteration: all their loads are issued before the first is consumed
+    int i = 0;
+    for (; i + 4 <= n_act; i += 4) {
+      float L[4];
+      f32x4 x0[4], x1[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t s = part_of(i + u);
+        L[u] = lse_row[s * lse_stride];
+        x0[u] = *(const f32x4*)(o_row + s * o_stride);
+        x1[u] = *(const f32x4*)(o_row + s * o_stride + 4);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float w = __expf(L[u] - mx);
+        if (L[u] == -INFINITY) continue;  // identity element: its O may hold anything
+        wsum += w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          acc[e] = __builtin_fmaf(w, x0[u][e], acc[e]);
+          acc[4 + e] = __builtin_fmaf(w, x1[u][e], acc[4 + e]);
+        }
+      }
+    }
+    for (; i < n_act; ++i) {
+      const int64_t s = part_of(i);
+      const float Ls = lse_row[s * lse_stride];
+      const float w = __expf(Ls - mx);
+      const f32x4 x0 = *(const f32x4*)(o_row + s * o_stride), x1 = *(const f32x4*)(o_row + s * o_stride + 4);
+      if (Ls == -INFINITY) continue;
       wsum += w;
-      const float* src = a.o_parts + (s * a.part_stride_rows + row) * D + c8 * 8;
-      const f32x4 x0 = *(const f32x4*)src, x1 = *(const f32x4*)(src + 4);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         acc[e] = __builtin_fmaf(w, x0[e], acc[e]);
