@@ -24,7 +24,7 @@ PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0}
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per block-kernel launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
 # see profiles/; None where not measured for that workload.
-MEASURED_TRAFFIC = {"cfg4": 7.61e8}   # 456.9 MB fetched + 304.3 MB written, average over the 8 launches of a step
+MEASURED_TRAFFIC = {"cfg4": 7.82e8}   # 465.1 MB fetched + 316.9 MB written, average over the 8 launches of a step
 
 
 def describe(w):
