@@ -72,35 +72,48 @@ int validate(const ringattn_params* p, Derived* d) {
 
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
+constexpr int kMaxGroups = 8;  // launches per forward
+
 size_t workspace_bytes_of(const ringattn_params* p, const Derived& d) {
   return (size_t)p->npes * (size_t)d.rows * (size_t)(p->dim + 1) * sizeof(float);
 }
 
 }  // namespace
 
+// One launch of the forward: the (rank, step) pairs of a few virtual ranks, all their steps.
+struct LaunchGroup {
+  int pair_begin, pair_count;  // slice of the pair table
+  int rank_begin, rank_count;  // slice of group_ranks
+};
+
 struct ringattn_plan {
-  ringattn_params p;
-  int seqlen[RINGATTN_MAX_NPES];
-  Derived d;
-  void* ws;
-  size_t ws_bytes;
-  bool own_ws;
-  float* o_parts;    // [npes, rows, dim]
-  float* lse_parts;  // [npes, rows]
-  // Ring steps write disjoint partial slots, so for short chunks consecutive steps are issued
-  // round-robin on the caller's stream and two forked streams: the tail of one launch
-  // overlaps the head of the next.  Created lazily at the first forward (default priority).
-  hipStream_t aux[2];
-  hipEvent_t ev_fork;
-  hipEvent_t ev_join[2];
-  bool streams_ready;
+  ringattn_params p{};
+  int seqlen[RINGATTN_MAX_NPES]{};
+  Derived d{};
+  void* ws = nullptr;
+  size_t ws_bytes = 0;
+  bool own_ws = false;
+  float* o_parts = nullptr;    // [npes, rows, dim]
+  float* lse_parts = nullptr;  // [npes, rows]
+  // Launch schedule of ringattn_fwd.  The ring steps of different ranks are independent
+  // (each (rank, step) pair writes its own rows of its step's partial slot), so the forward
+  // is issued as a few launches that each hold ALL steps of a few ranks; the merge of those
+  // ranks then runs on a second stream underneath the next launch.
+  std::vector<int> h_pairs;       // packed (rank << 16 | step), launch by launch
+  std::vector<int> group_ranks;
+  std::vector<LaunchGroup> groups;
+  int* d_pairs = nullptr;         // device copy of h_pairs (allocated at the first forward)
+  hipStream_t merge_stream = nullptr;
+  hipEvent_t ev_group[kMaxGroups]{};
+  hipEvent_t ev_done = nullptr;
+  bool streams_ready = false;
   // hipGraph replay (RINGATTN_FLAG_GRAPH): one captured graph per pointer set
-  hipStream_t cap_stream;
-  hipGraph_t graph;
-  hipGraphExec_t exec;
-  const void *gq, *gk, *gv;
-  void* gout;
-  float* glse;
+  hipStream_t cap_stream = nullptr;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  const void *gq = nullptr, *gk = nullptr, *gv = nullptr;
+  void* gout = nullptr;
+  float* glse = nullptr;
 };
 
 namespace {
@@ -129,6 +142,8 @@ int launch_step(const ringattn_plan* pl, int s, const void* q, const void* k, co
   a.S = (int)pl->d.S;
   a.chunk = pl->d.chunk;
   a.P = pl->p.npes;
+  a.pairs = nullptr;
+  a.part_stride_rows = 0;
   a.step = s;
   active_ranks(pl->p.npes, pl->p.causal, s, &a.rank_base, &a.n_active);
   a.BH = (int)pl->d.BH;
@@ -139,65 +154,129 @@ int launch_step(const ringattn_plan* pl, int s, const void* q, const void* k, co
 }
 
 int launch_ring_merge(const ringattn_plan* pl, const float* o_parts, const float* lse_parts, void* out,
-                      float* lse, hipStream_t stream) {
+                      float* lse, hipStream_t stream, int rank_sel = -1) {
   ringattn::MergeArgs m;
   m.o_parts = o_parts;
   m.lse_parts = lse_parts;
   m.out = out;
   m.lse = lse;
-  m.rows = pl->d.rows;
+  m.rows = rank_sel >= 0 ? pl->d.BH * pl->d.chunk : pl->d.rows;
   m.part_stride_rows = pl->d.rows;
   m.n_parts = pl->p.npes;
   m.causal_ring = pl->p.causal ? 1 : 0;
   m.S = (int)pl->d.S;
   m.chunk = pl->d.chunk;
   m.P = pl->p.npes;
+  m.rank_sel = rank_sel;
   RA_HIP(ringattn::launch_merge(m, pl->p.dtype, pl->p.dim, stream));
   return RINGATTN_OK;
 }
 
-constexpr int kAuxStreams = 2;
-constexpr int kForkMaxChunk = 1024;
+// Launch schedule.  Causal: rank r has r + 1 visible chunks, so ranks are paired (P-1-g, g)
+// to give every launch the same work; non-causal: consecutive ranks.  At most kMaxGroups
+// launches.  Within a launch the pairs of one rank are listed in ring order
+// (csrc/ring_attention.cu:456-470: step s visits chunk (r + s) mod P).
+void build_schedule(ringattn_plan* pl) {
+  const int P = pl->p.npes;
+  const bool causal = pl->p.causal != 0;
+  std::vector<int> order;  // ranks in launch order
+  if (causal) {
+    for (int g = 0; g < (P + 1) / 2; ++g) {
+      order.push_back(P - 1 - g);
+      if (g != P - 1 - g) order.push_back(g);
+    }
+  } else {
+    for (int r = 0; r < P; ++r) order.push_back(r);
+  }
+  const int n_groups = P < 4 ? 1 : (P / 2 < kMaxGroups ? (causal ? (P + 1) / 2 : (P < 8 ? P / 2 : 4)) : (causal ? kMaxGroups : 4));
+  size_t pos = 0;
+  for (int g = 0; g < n_groups; ++g) {
+    // even split of the rank list; causal lists come in balanced pairs, keep pairs together
+    size_t end = (size_t)order.size() * (g + 1) / n_groups;
+    if (causal && (end & 1) && end < order.size()) ++end;
+    if (g == n_groups - 1) end = order.size();
+    if (end <= pos) continue;
+    LaunchGroup lg;
+    lg.pair_begin = (int)pl->h_pairs.size();
+    lg.rank_begin = (int)pl->group_ranks.size();
+    for (size_t i = pos; i < end; ++i) {
+      const int r = order[i];
+      pl->group_ranks.push_back(r);
+      for (int s = 0; s < P; ++s) {
+        const int j = (r + s) % P;
+        if (!causal || j <= r) pl->h_pairs.push_back((r << 16) | s);
+      }
+    }
+    lg.pair_count = (int)pl->h_pairs.size() - lg.pair_begin;
+    lg.rank_count = (int)pl->group_ranks.size() - lg.rank_begin;
+    pl->groups.push_back(lg);
+    pos = end;
+  }
+}
 
 int ensure_streams(ringattn_plan* pl) {
   if (pl->streams_ready) return RINGATTN_OK;
-  for (int i = 0; i < kAuxStreams; ++i) {
-    RA_HIP(hipStreamCreateWithFlags(&pl->aux[i], hipStreamNonBlocking));
-    RA_HIP(hipEventCreateWithFlags(&pl->ev_join[i], hipEventDisableTiming));
-  }
-  RA_HIP(hipEventCreateWithFlags(&pl->ev_fork, hipEventDisableTiming));
+  RA_HIP(hipMalloc((void**)&pl->d_pairs, pl->h_pairs.size() * sizeof(int)));
+  RA_HIP(hipMemcpy(pl->d_pairs, pl->h_pairs.data(), pl->h_pairs.size() * sizeof(int), hipMemcpyHostToDevice));
+  RA_HIP(hipStreamCreateWithFlags(&pl->merge_stream, hipStreamNonBlocking));
+  for (int i = 0; i < kMaxGroups; ++i) RA_HIP(hipEventCreateWithFlags(&pl->ev_group[i], hipEventDisableTiming));
+  RA_HIP(hipEventCreateWithFlags(&pl->ev_done, hipEventDisableTiming));
   pl->streams_ready = true;
   return RINGATTN_OK;
 }
 
-// The ring step loop (csrc/ring_attention.cu:456-620 moved to the host) plus the merge.
-// Steps are independent (each writes its own partial slot), so they are spread over the
-// caller's stream and the forked streams; the merge waits for all of them.
+int launch_group(const ringattn_plan* pl, const LaunchGroup& lg, const void* q, const void* k, const void* v,
+                 hipStream_t stream) {
+  ringattn::BlockStepArgs a;
+  a.q = q;
+  a.k = k;
+  a.v = v;
+  a.o_part = pl->o_parts;
+  a.lse_part = pl->lse_parts;
+  a.bh_stride = pl->d.S * pl->p.dim;
+  a.S = (int)pl->d.S;
+  a.chunk = pl->d.chunk;
+  a.P = pl->p.npes;
+  a.pairs = pl->d_pairs + lg.pair_begin;
+  a.part_stride_rows = pl->d.rows;
+  a.step = 0;
+  a.rank_base = 0;
+  a.n_active = lg.pair_count;
+  a.BH = (int)pl->d.BH;
+  a.causal = pl->p.causal ? 1 : 0;
+  a.scale_log2 = pl->d.scale * 1.4426950408889634f;
+  RA_HIP(ringattn::launch_block_step(a, pl->p.dtype, pl->p.dim, stream));
+  return RINGATTN_OK;
+}
+
+// The ring step loop (csrc/ring_attention.cu:456-620 moved to the host) plus the merge:
+// for every launch group, all ring steps of its ranks, then the merge of those ranks'
+// rows on the merge stream while the next group computes.  The last group's merge runs
+// on the caller's stream, which finally waits for the merge stream.
 int run_forward(ringattn_plan* pl, const void* q, const void* k, const void* v, void* out,
                 float* lse, hipStream_t stream) {
-  const int P = pl->p.npes;
-  // Forking pays for short launches (small chunks), where launch tails dominate; with long
-  // chunks concurrent launches disturb the lockstep of the q tiles that share a KV chunk in
-  // L2 and cost more than the tails they hide (measured: +4..7 % at chunk <= 1024, -2.5 % at 4096).
-  const int n_aux = (P > 1 && pl->d.chunk <= kForkMaxChunk) ? kAuxStreams : 0;
-  if (n_aux) {
-    int rc = ensure_streams(pl);
+  int rc = RINGATTN_OK;
+  const size_t G = pl->groups.size();
+  for (size_t g = 0; g < G; ++g) {
+    const LaunchGroup& lg = pl->groups[g];
+    rc = launch_group(pl, lg, q, k, v, stream);
     if (rc != RINGATTN_OK) return rc;
-    RA_HIP(hipEventRecord(pl->ev_fork, stream));
-    for (int i = 0; i < n_aux; ++i) RA_HIP(hipStreamWaitEvent(pl->aux[i], pl->ev_fork, 0));
+    hipStream_t ms = stream;
+    if (g + 1 < G) {
+      RA_HIP(hipEventRecord(pl->ev_group[g], stream));
+      RA_HIP(hipStreamWaitEvent(pl->merge_stream, pl->ev_group[g], 0));
+      ms = pl->merge_stream;
+    }
+    for (int i = 0; i < lg.rank_count; ++i) {
+      rc = launch_ring_merge(pl, pl->o_parts, pl->lse_parts, out, lse, ms, pl->group_ranks[lg.rank_begin + i]);
+      if (rc != RINGATTN_OK) return rc;
+    }
   }
-  for (int s = 0; s < P; ++s) {
-    const int lane = s % (n_aux + 1);
-    hipStream_t st = lane == 0 ? stream : pl->aux[lane - 1];
-    int rc = launch_step(pl, s, q, k, v, pl->o_parts + (size_t)s * pl->d.rows * pl->p.dim,
-                         pl->lse_parts + (size_t)s * pl->d.rows, st);
-    if (rc != RINGATTN_OK) return rc;
+  if (G > 1) {
+    RA_HIP(hipEventRecord(pl->ev_done, pl->merge_stream));
+    RA_HIP(hipStreamWaitEvent(stream, pl->ev_done, 0));
   }
-  for (int i = 0; i < n_aux; ++i) {
-    RA_HIP(hipEventRecord(pl->ev_join[i], pl->aux[i]));
-    RA_HIP(hipStreamWaitEvent(stream, pl->ev_join[i], 0));
-  }
-  return launch_ring_merge(pl, pl->o_parts, pl->lse_parts, out, lse, stream);
+  return RINGATTN_OK;
 }
 
 void drop_graph(ringattn_plan* pl) {
@@ -237,7 +316,6 @@ int ringattn_plan_create(const ringattn_params* params, void* workspace, size_t 
   }
   ringattn_plan* pl = new (std::nothrow) ringattn_plan();
   if (!pl) return RINGATTN_ERR_ALLOC;
-  std::memset(pl, 0, sizeof(*pl));
   pl->p = *params;
   std::memcpy(pl->seqlen, params->h_seqlen, sizeof(int) * (size_t)params->npes);
   pl->p.h_seqlen = pl->seqlen;
@@ -257,6 +335,7 @@ int ringattn_plan_create(const ringattn_params* params, void* workspace, size_t 
   }
   pl->o_parts = (float*)pl->ws;
   pl->lse_parts = pl->o_parts + (size_t)params->npes * d.rows * params->dim;
+  build_schedule(pl);
   {
     std::lock_guard<std::mutex> lk(g_plans_mu);
     g_plans.insert(pl);
@@ -274,11 +353,10 @@ int ringattn_plan_destroy(ringattn_plan* plan) {
   drop_graph(plan);
   if (plan->cap_stream) (void)hipStreamDestroy(plan->cap_stream);
   if (plan->streams_ready) {
-    for (int i = 0; i < kAuxStreams; ++i) {
-      (void)hipStreamDestroy(plan->aux[i]);
-      (void)hipEventDestroy(plan->ev_join[i]);
-    }
-    (void)hipEventDestroy(plan->ev_fork);
+    (void)hipStreamDestroy(plan->merge_stream);
+    for (int i = 0; i < kMaxGroups; ++i) (void)hipEventDestroy(plan->ev_group[i]);
+    (void)hipEventDestroy(plan->ev_done);
+    (void)hipFree(plan->d_pairs);
   }
   if (plan->own_ws && plan->ws) {
     hipError_t e = hipFree(plan->ws);
@@ -294,6 +372,9 @@ int ringattn_fwd(ringattn_plan* plan, const void* q, const void* k, const void* 
   if (!q || !k || !v || !out || !lse) return RINGATTN_ERR_NULL;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || ((uintptr_t)lse & 3u)) return RINGATTN_ERR_ALIGN;
   hipStream_t stream = (hipStream_t)stream_;
+  // pair table, merge stream and events: created at the first forward, outside any capture
+  int rc0 = ensure_streams(plan);
+  if (rc0 != RINGATTN_OK) return rc0;
   if (!(plan->p.flags & RINGATTN_FLAG_GRAPH)) return run_forward(plan, q, k, v, out, lse, stream);
 
   // hipGraph replay: the P + 1 launches are captured once per pointer set on a private
@@ -363,6 +444,7 @@ int ringattn_merge(const float* o_parts, const float* lse_parts, int n_parts, in
   m.S = 1;
   m.chunk = 1;
   m.P = n_parts;
+  m.rank_sel = -1;
   RA_HIP(ringattn::launch_merge(m, dtype, dim, (hipStream_t)stream));
   return RINGATTN_OK;
 }
@@ -418,6 +500,8 @@ int ringattn_ring_attention(const void* q, const void* k, const void* v, void* o
     a.S = (int)d.S;
     a.chunk = d.chunk;
     a.P = npes;
+    a.pairs = nullptr;
+    a.part_stride_rows = 0;
     a.step = steps[i];
     a.rank_base = mype;
     a.n_active = 1;

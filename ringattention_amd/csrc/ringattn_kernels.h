@@ -8,9 +8,14 @@ namespace ringattn {
 
 constexpr int kBlockM = 128;  // query rows per workgroup (4 waves x 32 rows)
 
-// One ring step for every active virtual rank: rank r = rank_base + ridx works on
-// KV chunk (r + step) mod P.  This is the launch-level restatement of the step loop
-// body of the reference kernel (csrc/ring_attention.cu:456-470,531-610).
+// A batch of (rank, ring step) pairs: rank r at step s works on KV chunk (r + s) mod P --
+// the launch-level restatement of the step loop body of the reference kernel
+// (csrc/ring_attention.cu:456-470,531-610).  Two ways to name the pairs:
+//   pairs == nullptr : one ring step for the ranks rank_base .. rank_base + n_active - 1;
+//                      o_part / lse_part point at that step's slot;
+//   pairs != nullptr : n_active packed pairs (rank << 16 | step) read from device memory;
+//                      o_part / lse_part point at slot 0 and step s is written at
+//                      + s * part_stride_rows rows.
 struct BlockStepArgs {
   const void* q;       // [BH, S, D] storage dtype
   const void* k;       // [BH, S, D]
@@ -21,9 +26,11 @@ struct BlockStepArgs {
   int S;               // tokens per head
   int chunk;           // tokens per virtual rank
   int P;               // virtual ranks
-  int step;            // ring step s
-  int rank_base;       // first active rank of this step
-  int n_active;        // active ranks in this step
+  const int* pairs;    // device array of packed (rank, step) pairs, or nullptr
+  int64_t part_stride_rows;  // rows between the partial slots of consecutive steps
+  int step;            // ring step s (pairs == nullptr)
+  int rank_base;       // first active rank of this step (pairs == nullptr)
+  int n_active;        // active ranks of the step, or number of pairs
   int BH;              // batch * heads
   int causal;          // chunk-level causal ring: j<r full, j==r diagonal mask
   float scale_log2;    // softmax_scale * log2(e)
@@ -42,6 +49,9 @@ struct MergeArgs {
   // is active iff s == 0 or r + s >= P; inactive parts are never read.
   int causal_ring;
   int S, chunk, P;
+  // rank_sel >= 0: only the rows of that virtual rank are merged (rows = BH * chunk, row i
+  // is row (i / chunk) * S + rank_sel * chunk + i % chunk of the tensors); -1: all rows.
+  int rank_sel;
 };
 
 // dtype: 0 = fp16, 1 = bf16.  Return hipSuccess or the launch error.

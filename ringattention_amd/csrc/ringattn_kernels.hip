@@ -144,8 +144,13 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   const int group = (slot / q_tiles) * 8 + xcd;
   if (group >= groups) return;
   const int ridx = group % a.n_active, bh = group / a.n_active;
-  const int r = a.rank_base + ridx;
-  int j = r + a.step;
+  int r = a.rank_base + ridx, step = a.step;
+  if (a.pairs) {
+    const int pr = a.pairs[ridx];
+    r = pr >> 16;
+    step = pr & 0xffff;
+  }
+  int j = r + step;
   if (j >= a.P) j -= a.P;
   if (a.causal && j > r) return;
   const bool diag = a.causal && (j == r);
@@ -416,7 +421,8 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
     const float l = cross_half_sum((ls[qb][0] + ls[qb][1]) + (ls[qb][2] + ls[qb][3]));
     const float inv = (l > 0.f) ? 1.f / l : 0.f;
     const int row_g = r * a.chunk + qt * BM + 32 * QB * wave + 32 * qb + n;
-    float* orow = a.o_part + ((int64_t)bh * a.S + row_g) * D;
+    const int64_t slot_rows = a.pairs ? (int64_t)step * a.part_stride_rows : 0;
+    float* orow = a.o_part + (slot_rows + (int64_t)bh * a.S + row_g) * D;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -428,7 +434,7 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
       }
     if (h == 0) {
       const float lse = (l > 0.f) ? (ms[qb] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
-      a.lse_part[(int64_t)bh * a.S + row_g] = lse;
+      a.lse_part[slot_rows + (int64_t)bh * a.S + row_g] = lse;
     }
   }
 }
@@ -456,8 +462,9 @@ template <int DT, int D>
 __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
   constexpr int TPR = D / 8;  // threads per row, 8 columns each
   constexpr int ROWS = 256 / TPR;
-  const int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / TPR;
+  int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / TPR;
   if (row >= a.rows) return;
+  if (a.rank_sel >= 0) row = (row / a.chunk) * a.S + (int64_t)a.rank_sel * a.chunk + row % a.chunk;
   const int c8 = threadIdx.x % TPR;
   // active parts of this row: part 0 and parts first_wrapped .. n_parts-1 (ring), or all
   int first_wrapped = 1;
