@@ -11,8 +11,8 @@
  *
  * Layout: Q, K, V, O are [batch, heads, S, dim] row-major, so each (batch, head)
  * slab is the reference's [seqlen, dim] layout (csrc/ring_attention.cu:422-426).
- * The sequence is split into npes chunks in order; virtual ring rank r owns rows
- * [r*c, (r+1)*c).  At ring step s rank r works on KV chunk (r + s) mod npes
+ * The sequence is split into npes chunks in order; virtual ring rank r owns the
+ * h_seqlen[r] rows that follow those of rank r-1.  At ring step s rank r works on KV chunk (r + s) mod npes
  * (csrc/ring_attention.cu:463,531,615) -- by indexing, no data is moved.
  */
 #ifndef RINGATTN_H
@@ -30,7 +30,7 @@ extern "C" {
 #define RINGATTN_ERR_NPES 2        /* npes < 1 or above RINGATTN_MAX_NPES */
 #define RINGATTN_ERR_DIM 3         /* dim not in {64, 128} */
 #define RINGATTN_ERR_DTYPE 4       /* dtype not fp16 / bf16 */
-#define RINGATTN_ERR_SEQLEN 5      /* chunk lengths not equal, not positive, or not a multiple of 128 */
+#define RINGATTN_ERR_SEQLEN 5      /* a per-rank length is not a positive multiple of 128, or max_seq is below it */
 #define RINGATTN_ERR_SHAPE 6       /* batch or heads < 1, sizes overflow */
 #define RINGATTN_ERR_WORKSPACE 7   /* caller workspace missing or too small */
 #define RINGATTN_ERR_RANK 8        /* mype / step outside [0, npes) */
@@ -43,7 +43,7 @@ extern "C" {
 #define RINGATTN_DTYPE_BF16 1
 
 #define RINGATTN_MAX_NPES 64
-#define RINGATTN_TILE 128          /* chunk lengths must be multiples of this */
+#define RINGATTN_TILE 128          /* per-rank lengths must be multiples of this; they may differ between ranks */
 
 #define RINGATTN_FLAG_GRAPH 1      /* capture the step loop + merge in a hipGraph and replay it */
 
@@ -57,7 +57,8 @@ extern "C" {
  */
 typedef struct ringattn_params {
   int npes;              /* P: virtual ring ranks */
-  const int* h_seqlen;   /* [npes] tokens per rank (host array, read during the call only) */
+  const int* h_seqlen;   /* [npes] tokens per rank, may differ per rank like the reference's seqlen[]
+                            (csrc/ring_attention.cu:753); host array, read during the call only */
   int dim;               /* head dimension: 64 or 128 */
   float softmax_scale;   /* logit scale; <= 0 selects 1/sqrt(dim) */
   int batch;

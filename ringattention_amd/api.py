@@ -51,13 +51,18 @@ class RingAttention:
     """A forward plan for P virtual ring ranks on one GPU."""
 
     def __init__(self, npes, chunk, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, graph=False):
+        """`chunk`: tokens per rank -- one int for equal chunks or a list of npes lengths
+        (the per-PE seqlen[] of csrc/ring_attention.cu:753)."""
         self.lib = _lib.load()
+        self.seqlen = [int(chunk)] * npes if isinstance(chunk, int) else [int(x) for x in chunk]
+        if len(self.seqlen) != npes:
+            raise ValueError("need one length per rank")
         self.npes, self.chunk, self.dim, self.batch, self.heads = npes, chunk, dim, batch, heads
         self.dtype_code = DTYPE_CODE[dtype]
         self.torch_dtype = TORCH_DTYPE[self.dtype_code]
         self.causal = bool(causal)
-        self.seq = npes * chunk
-        self.params = make_params(npes, [chunk] * npes, dim, batch, heads, dtype, causal, softmax_scale,
+        self.seq = sum(self.seqlen)
+        self.params = make_params(npes, self.seqlen, dim, batch, heads, dtype, causal, softmax_scale,
                                   FLAG_GRAPH if graph else 0)
         self.handle = ctypes.c_void_p()
         check(self.lib.ringattn_plan_create(ctypes.byref(self.params), None, 0, ctypes.byref(self.handle)),

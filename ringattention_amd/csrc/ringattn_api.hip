@@ -33,7 +33,8 @@ inline int hip_fail(hipError_t e) {
   } while (0)
 
 struct Derived {
-  int chunk = 0;
+  int start[RINGATTN_MAX_NPES + 1] = {};  // rank r owns rows [start[r], start[r+1]) of every head
+  int max_len = 0;
   int64_t S = 0;
   int64_t BH = 0;
   int64_t rows = 0;  // BH * S
@@ -50,18 +51,23 @@ int validate(const ringattn_params* p, Derived* d) {
   if (p->dim != 64 && p->dim != 128) return RINGATTN_ERR_DIM;
   if (p->dtype != RINGATTN_DTYPE_FP16 && p->dtype != RINGATTN_DTYPE_BF16) return RINGATTN_ERR_DTYPE;
   if (p->batch < 1 || p->heads < 1) return RINGATTN_ERR_SHAPE;
-  const int c = p->h_seqlen[0];
-  if (c <= 0 || c % RINGATTN_TILE != 0) return RINGATTN_ERR_SEQLEN;
-  for (int r = 1; r < p->npes; ++r)
-    if (p->h_seqlen[r] != c) return RINGATTN_ERR_SEQLEN;
-  const int64_t S = (int64_t)c * p->npes;
+  int64_t S = 0;
+  int max_len = 0;
+  for (int r = 0; r < p->npes; ++r) {
+    const int c = p->h_seqlen[r];
+    if (c <= 0 || c % RINGATTN_TILE != 0) return RINGATTN_ERR_SEQLEN;
+    S += c;
+    if (c > max_len) max_len = c;
+  }
   const int64_t BH = (int64_t)p->batch * p->heads;
   if (S > INT32_MAX / 2 || BH > INT32_MAX / 2) return RINGATTN_ERR_SHAPE;
   if (BH * p->npes > (int64_t)INT32_MAX / 64) return RINGATTN_ERR_SHAPE;  // grid size
   if (BH * S > (int64_t)1 << 40) return RINGATTN_ERR_SHAPE;
   if (!std::isfinite(p->softmax_scale)) return RINGATTN_ERR_SHAPE;
   if (d) {
-    d->chunk = c;
+    d->start[0] = 0;
+    for (int r = 0; r < p->npes; ++r) d->start[r + 1] = d->start[r] + p->h_seqlen[r];
+    d->max_len = max_len;
     d->S = S;
     d->BH = BH;
     d->rows = BH * S;
@@ -130,44 +136,51 @@ inline void active_ranks(int P, int causal, int s, int* rank_base, int* n_active
   }
 }
 
+// fields of the launch arguments that depend only on the geometry
+void fill_geometry(ringattn::BlockStepArgs& a, const ringattn_params& p, const Derived& d) {
+  a.bh_stride = d.S * p.dim;
+  a.S = (int)d.S;
+  a.q_tiles_max = d.max_len / ringattn::kBlockM;
+  a.P = p.npes;
+  a.BH = (int)d.BH;
+  a.causal = p.causal ? 1 : 0;
+  a.scale_log2 = d.scale * 1.4426950408889634f;
+  for (int r = 0; r <= p.npes; ++r) a.rank_start[r] = d.start[r];
+}
+
 int launch_step(const ringattn_plan* pl, int s, const void* q, const void* k, const void* v,
                 float* o_part, float* lse_part, hipStream_t stream) {
   ringattn::BlockStepArgs a;
+  fill_geometry(a, pl->p, pl->d);
   a.q = q;
   a.k = k;
   a.v = v;
   a.o_part = o_part;
   a.lse_part = lse_part;
-  a.bh_stride = pl->d.S * pl->p.dim;
-  a.S = (int)pl->d.S;
-  a.chunk = pl->d.chunk;
-  a.P = pl->p.npes;
   a.pairs = nullptr;
   a.part_stride_rows = 0;
   a.step = s;
   active_ranks(pl->p.npes, pl->p.causal, s, &a.rank_base, &a.n_active);
-  a.BH = (int)pl->d.BH;
-  a.causal = pl->p.causal ? 1 : 0;
-  a.scale_log2 = pl->d.scale * 1.4426950408889634f;
   RA_HIP(ringattn::launch_block_step(a, pl->p.dtype, pl->p.dim, stream));
   return RINGATTN_OK;
 }
 
-int launch_ring_merge(const ringattn_plan* pl, const float* o_parts, const float* lse_parts, void* out,
-                      float* lse, hipStream_t stream, int rank_sel = -1) {
+// merge of the rows of one virtual rank; with a causal ring, part s of rank r is active iff
+// s == 0 or r + s >= P, and inactive parts are never read
+int launch_rank_merge(const ringattn_plan* pl, const float* o_parts, const float* lse_parts, void* out,
+                      float* lse, hipStream_t stream, int rank) {
   ringattn::MergeArgs m;
   m.o_parts = o_parts;
   m.lse_parts = lse_parts;
   m.out = out;
   m.lse = lse;
-  m.rows = rank_sel >= 0 ? pl->d.BH * pl->d.chunk : pl->d.rows;
+  m.sel_start = pl->d.start[rank];
+  m.sel_len = pl->d.start[rank + 1] - pl->d.start[rank];
+  m.rows = pl->d.BH * m.sel_len;
   m.part_stride_rows = pl->d.rows;
   m.n_parts = pl->p.npes;
-  m.causal_ring = pl->p.causal ? 1 : 0;
+  m.first_wrapped = pl->p.causal ? pl->p.npes - rank : 1;
   m.S = (int)pl->d.S;
-  m.chunk = pl->d.chunk;
-  m.P = pl->p.npes;
-  m.rank_sel = rank_sel;
   RA_HIP(ringattn::launch_merge(m, pl->p.dtype, pl->p.dim, stream));
   return RINGATTN_OK;
 }
@@ -228,23 +241,17 @@ int ensure_streams(ringattn_plan* pl) {
 int launch_group(const ringattn_plan* pl, const LaunchGroup& lg, const void* q, const void* k, const void* v,
                  hipStream_t stream) {
   ringattn::BlockStepArgs a;
+  fill_geometry(a, pl->p, pl->d);
   a.q = q;
   a.k = k;
   a.v = v;
   a.o_part = pl->o_parts;
   a.lse_part = pl->lse_parts;
-  a.bh_stride = pl->d.S * pl->p.dim;
-  a.S = (int)pl->d.S;
-  a.chunk = pl->d.chunk;
-  a.P = pl->p.npes;
   a.pairs = pl->d_pairs + lg.pair_begin;
   a.part_stride_rows = pl->d.rows;
   a.step = 0;
   a.rank_base = 0;
   a.n_active = lg.pair_count;
-  a.BH = (int)pl->d.BH;
-  a.causal = pl->p.causal ? 1 : 0;
-  a.scale_log2 = pl->d.scale * 1.4426950408889634f;
   RA_HIP(ringattn::launch_block_step(a, pl->p.dtype, pl->p.dim, stream));
   return RINGATTN_OK;
 }
@@ -268,7 +275,7 @@ int run_forward(ringattn_plan* pl, const void* q, const void* k, const void* v, 
       ms = pl->merge_stream;
     }
     for (int i = 0; i < lg.rank_count; ++i) {
-      rc = launch_ring_merge(pl, pl->o_parts, pl->lse_parts, out, lse, ms, pl->group_ranks[lg.rank_begin + i]);
+      rc = launch_rank_merge(pl, pl->o_parts, pl->lse_parts, out, lse, ms, pl->group_ranks[lg.rank_begin + i]);
       if (rc != RINGATTN_OK) return rc;
     }
   }
@@ -421,7 +428,11 @@ int ringattn_merge_ring(ringattn_plan* plan, const float* o_parts, const float* 
   if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
   if (!o_parts || !lse_parts || !out || !lse) return RINGATTN_ERR_NULL;
   if (!aligned16(o_parts) || !aligned16(out) || ((uintptr_t)lse_parts & 3u) || ((uintptr_t)lse & 3u)) return RINGATTN_ERR_ALIGN;
-  return launch_ring_merge(plan, o_parts, lse_parts, out, lse, (hipStream_t)stream);
+  for (int r = 0; r < plan->p.npes; ++r) {
+    int rc = launch_rank_merge(plan, o_parts, lse_parts, out, lse, (hipStream_t)stream, r);
+    if (rc != RINGATTN_OK) return rc;
+  }
+  return RINGATTN_OK;
 }
 
 int ringattn_merge(const float* o_parts, const float* lse_parts, int n_parts, int64_t rows, int dim,
@@ -440,11 +451,10 @@ int ringattn_merge(const float* o_parts, const float* lse_parts, int n_parts, in
   m.rows = rows;
   m.part_stride_rows = rows;
   m.n_parts = n_parts;
-  m.causal_ring = 0;
-  m.S = 1;
-  m.chunk = 1;
-  m.P = n_parts;
-  m.rank_sel = -1;
+  m.first_wrapped = 1;
+  m.S = (int)(rows > 0 ? (rows < INT32_MAX ? rows : INT32_MAX) : 1);
+  m.sel_start = 0;
+  m.sel_len = m.S;
   RA_HIP(ringattn::launch_merge(m, dtype, dim, (hipStream_t)stream));
   return RINGATTN_OK;
 }
@@ -466,7 +476,7 @@ int ringattn_ring_attention(const void* q, const void* k, const void* v, void* o
   int rc = validate(&p, &d);
   if (rc != RINGATTN_OK) return rc;
   if (mype < 0 || mype >= npes) return RINGATTN_ERR_RANK;
-  if (max_seq < d.chunk) return RINGATTN_ERR_SEQLEN;
+  if (max_seq < d.max_len) return RINGATTN_ERR_SEQLEN;
   if (!q || !k || !v || !out) return RINGATTN_ERR_NULL;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return RINGATTN_ERR_ALIGN;
 
@@ -477,7 +487,8 @@ int ringattn_ring_attention(const void* q, const void* k, const void* v, void* o
     if (!causal || j <= mype) steps.push_back(s);
   }
   const int n_parts = (int)steps.size();
-  const size_t c = (size_t)d.chunk;
+  const size_t c = (size_t)(d.start[mype + 1] - d.start[mype]);  // rows of this rank
+  const size_t first = (size_t)d.start[mype];
   // per-call scratch, like the reference's per-call allocations (:383-394) but freed
   float* ws = nullptr;
   RA_HIP(hipMalloc((void**)&ws, (size_t)n_parts * c * (size_t)(dim + 1) * sizeof(float) + c * sizeof(float)));
@@ -485,29 +496,23 @@ int ringattn_ring_attention(const void* q, const void* k, const void* v, void* o
   float* lse_parts = ws + (size_t)n_parts * c * dim;
   float* lse_tmp = lse_parts + (size_t)n_parts * c;
   const size_t esz = 2;
-  // The kernel addresses rows of rank r at r * chunk: shift the rank-local buffers so
-  // that rank mype's rows land on them.  The shifted pointers are never dereferenced
-  // outside [mype * chunk, (mype + 1) * chunk).
-  const char* q_shift = (const char*)q - (size_t)mype * c * dim * esz;
+  // The kernel addresses the rows of rank r at rank_start[r]: shift the rank-local buffers
+  // so that rank mype's rows land on them.  The shifted pointers are never dereferenced
+  // outside [start[mype], start[mype + 1]).
+  const char* q_shift = (const char*)q - first * dim * esz;
   for (int i = 0; i < n_parts && rc == RINGATTN_OK; ++i) {
     ringattn::BlockStepArgs a;
+    fill_geometry(a, p, d);
     a.q = q_shift;
     a.k = k;
     a.v = v;
-    a.o_part = o_parts + (size_t)i * c * dim - (size_t)mype * c * dim;
-    a.lse_part = lse_parts + (size_t)i * c - (size_t)mype * c;
-    a.bh_stride = d.S * dim;
-    a.S = (int)d.S;
-    a.chunk = d.chunk;
-    a.P = npes;
+    a.o_part = o_parts + (size_t)i * c * dim - first * dim;
+    a.lse_part = lse_parts + (size_t)i * c - first;
     a.pairs = nullptr;
     a.part_stride_rows = 0;
     a.step = steps[i];
     a.rank_base = mype;
     a.n_active = 1;
-    a.BH = 1;
-    a.causal = causal ? 1 : 0;
-    a.scale_log2 = d.scale * 1.4426950408889634f;
     hipError_t e = ringattn::launch_block_step(a, dtype, dim, nullptr);
     if (e != hipSuccess) rc = hip_fail(e);
   }
@@ -525,7 +530,7 @@ const char* ringattn_strerror(int code) {
     case RINGATTN_ERR_NPES: return "npes out of range";
     case RINGATTN_ERR_DIM: return "dim must be 64 or 128";
     case RINGATTN_ERR_DTYPE: return "dtype must be fp16 (0) or bf16 (1)";
-    case RINGATTN_ERR_SEQLEN: return "per-rank sequence lengths must be equal, positive multiples of 128";
+    case RINGATTN_ERR_SEQLEN: return "per-rank sequence lengths must be positive multiples of 128 (and max_seq at least the longest)";
     case RINGATTN_ERR_SHAPE: return "batch/heads/scale invalid or sizes overflow";
     case RINGATTN_ERR_WORKSPACE: return "workspace too small";
     case RINGATTN_ERR_RANK: return "rank or step outside [0, npes)";

@@ -7,6 +7,7 @@
 namespace ringattn {
 
 constexpr int kBlockM = 128;  // query rows per workgroup (4 waves x 32 rows)
+constexpr int kMaxRanks = 64;
 
 // A batch of (rank, ring step) pairs: rank r at step s works on KV chunk (r + s) mod P --
 // the launch-level restatement of the step loop body of the reference kernel
@@ -24,7 +25,7 @@ struct BlockStepArgs {
   float* lse_part;     // [BH, S]    fp32 partial LSE of this step (natural log)
   int64_t bh_stride;   // elements between heads (= S * D)
   int S;               // tokens per head
-  int chunk;           // tokens per virtual rank
+  int q_tiles_max;     // kBlockM-row q tiles of the longest rank (grid dimension)
   int P;               // virtual ranks
   const int* pairs;    // device array of packed (rank, step) pairs, or nullptr
   int64_t part_stride_rows;  // rows between the partial slots of consecutive steps
@@ -34,24 +35,25 @@ struct BlockStepArgs {
   int BH;              // batch * heads
   int causal;          // chunk-level causal ring: j<r full, j==r diagonal mask
   float scale_log2;    // softmax_scale * log2(e)
+  // rank r owns rows [rank_start[r], rank_start[r+1]) of every head; lengths are multiples
+  // of kBlockM and may differ per rank (the per-PE seqlen[] of csrc/ring_attention.cu:753)
+  int rank_start[kMaxRanks + 1];
 };
 
-// P-way merge of the per-step partials into the final O (storage dtype) and LSE.
+// n-way merge of (O, LSE) partials into the final O (storage dtype) and LSE, for the rows
+// [sel_start, sel_start + sel_len) of every head (one virtual rank, or everything).
 struct MergeArgs {
-  const float* o_parts;   // [n_parts, rows, D]
-  const float* lse_parts; // [n_parts, rows]
-  void* out;              // [rows, D] storage dtype
-  float* lse;             // [rows]
-  int64_t rows;           // BH * S
-  int64_t part_stride_rows;  // rows between consecutive parts (>= rows)
+  const float* o_parts;   // [n_parts, heads * S, D]
+  const float* lse_parts; // [n_parts, heads * S]
+  void* out;              // [heads * S, D] storage dtype
+  float* lse;             // [heads * S]
+  int64_t rows;           // heads * sel_len rows are merged
+  int64_t part_stride_rows;  // rows between consecutive parts (>= heads * S)
   int n_parts;
-  // ring structure: when causal_ring != 0, part s of a row of rank r = (row % S) / chunk
-  // is active iff s == 0 or r + s >= P; inactive parts are never read.
-  int causal_ring;
-  int S, chunk, P;
-  // rank_sel >= 0: only the rows of that virtual rank are merged (rows = BH * chunk, row i
-  // is row (i / chunk) * S + rank_sel * chunk + i % chunk of the tensors); -1: all rows.
-  int rank_sel;
+  int first_wrapped;      // active parts: part 0 and parts first_wrapped .. n_parts-1 (1 = all);
+                          // inactive parts are never read
+  int S;                  // rows per head
+  int sel_start, sel_len; // row range within a head
 };
 
 // dtype: 0 = fp16, 1 = bf16.  Return hipSuccess or the launch error.

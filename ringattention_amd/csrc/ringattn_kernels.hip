@@ -138,7 +138,7 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   const int n = lane & 31, h = lane >> 5;
 
   // workgroup -> (head, rank, q tile), XCD-aware as in block_attention_kernel
-  const int q_tiles = a.chunk / BM;
+  const int q_tiles = a.q_tiles_max;
   const int groups = a.n_active * a.BH;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int group = (slot / q_tiles) * 8 + xcd;
@@ -154,15 +154,18 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   if (j >= a.P) j -= a.P;
   if (a.causal && j > r) return;
   const bool diag = a.causal && (j == r);
+  const int q_start = a.rank_start[r], q_len = a.rank_start[r + 1] - q_start;
+  const int kv_start = a.rank_start[j], kv_len = a.rank_start[j + 1] - kv_start;
   int qt = slot % q_tiles;
-  if (diag) qt = q_tiles - 1 - qt;
-  const int n_tiles = diag ? ((qt + 1) * BM) / BN : a.chunk / BN;
+  if (qt * BM >= q_len) return;  // ranks shorter than the longest one
+  if (diag) qt = q_len / BM - 1 - qt;
+  const int n_tiles = diag ? ((qt + 1) * BM) / BN : kv_len / BN;
   const int first_masked = diag ? (qt * BM) / BN : n_tiles;  // tiles >= this need the causal mask
 
   const int64_t head_off = (int64_t)bh * a.bh_stride;
-  const char* qbase = (const char*)a.q + (head_off + (int64_t)(r * a.chunk + qt * BM) * D) * 2;
-  const char* kbase = (const char*)a.k + (head_off + (int64_t)j * a.chunk * D) * 2;
-  const char* vbase = (const char*)a.v + (head_off + (int64_t)j * a.chunk * D) * 2;
+  const char* qbase = (const char*)a.q + (head_off + (int64_t)(q_start + qt * BM) * D) * 2;
+  const char* kbase = (const char*)a.k + (head_off + (int64_t)kv_start * D) * 2;
+  const char* vbase = (const char*)a.v + (head_off + (int64_t)kv_start * D) * 2;
 
   // this lane's query rows (local to the q tile): 32 QB wave + 32 qb + n
   s16x8 qf[QB][KS];
@@ -420,7 +423,7 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   for (int qb = 0; qb < QB; ++qb) {
     const float l = cross_half_sum((ls[qb][0] + ls[qb][1]) + (ls[qb][2] + ls[qb][3]));
     const float inv = (l > 0.f) ? 1.f / l : 0.f;
-    const int row_g = r * a.chunk + qt * BM + 32 * QB * wave + 32 * qb + n;
+    const int row_g = q_start + qt * BM + 32 * QB * wave + 32 * qb + n;
     const int64_t slot_rows = a.pairs ? (int64_t)step * a.part_stride_rows : 0;
     float* orow = a.o_part + (slot_rows + (int64_t)bh * a.S + row_g) * D;
 #pragma unroll
@@ -464,14 +467,10 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
   constexpr int ROWS = 256 / TPR;
   int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / TPR;
   if (row >= a.rows) return;
-  if (a.rank_sel >= 0) row = (row / a.chunk) * a.S + (int64_t)a.rank_sel * a.chunk + row % a.chunk;
+  row = (row / a.sel_len) * a.S + a.sel_start + row % a.sel_len;
   const int c8 = threadIdx.x % TPR;
   // active parts of this row: part 0 and parts first_wrapped .. n_parts-1 (ring), or all
-  int first_wrapped = 1;
-  if (a.causal_ring) {
-    const int r = (int)((row % a.S) / a.chunk);
-    first_wrapped = a.P - r;
-  }
+  const int first_wrapped = a.first_wrapped;
   const int n_act = a.n_parts - first_wrapped + 1;
   auto part_of = [&](int i) { return i == 0 ? 0 : first_wrapped + i - 1; };
   const float* lse_row = a.lse_parts + row;
@@ -533,7 +532,7 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
 // ---- host launchers -----------------------------------------------------------------
 hipError_t launch_block_step(const BlockStepArgs& a, int dtype, int dim, hipStream_t stream) {
   if (a.n_active <= 0) return hipSuccess;
-  const int q_tiles = a.chunk / kBlockM;
+  const int q_tiles = a.q_tiles_max;
   const int groups = a.n_active * a.BH;
   const unsigned grid = (unsigned)(((groups + 7) / 8) * 8 * q_tiles);
   if (dtype == 0 && dim == 64) block_attention_kernel<0, 64><<<grid, 256, 0, stream>>>(a);

@@ -46,6 +46,7 @@ def test_header_constants_match_error_strings(ralib):
 def test_parameter_validation(ralib):
     wb = ralib.ringattn_workspace_bytes
     assert wb(ctypes.byref(params())) == 2 * 256 * 65 * 4
+    assert wb(ctypes.byref(params(seqlen=(128, 384)))) == 2 * 512 * 65 * 4   # unequal per-rank lengths are fine
     h = ctypes.c_void_p()
 
     def create(p):
@@ -63,8 +64,8 @@ def test_parameter_validation(ralib):
         assert create(params(dim=bad_dim)) == E_DIM
     assert create(params(dtype=2)) == E_DTYPE
     assert create(params(dtype=-1)) == E_DTYPE
-    assert create(params(seqlen=(128, 256))) == E_SEQLEN      # unequal chunks
-    assert create(params(seqlen=(100, 100))) == E_SEQLEN      # not a multiple of the tile
+    assert create(params(seqlen=(128, 200))) == E_SEQLEN      # one rank not a multiple of the tile
+    assert create(params(seqlen=(100, 100))) == E_SEQLEN
     assert create(params(seqlen=(0, 0))) == E_SEQLEN
     assert create(params(seqlen=(-128, -128))) == E_SEQLEN
     assert create(params(batch=0)) == E_SHAPE

@@ -111,6 +111,45 @@ def test_shapes_and_edges_full(oracle, w):
     check_rows(oracle, w, q, k, v, out, lse, np.arange(w.rows))
 
 
+@pytest.mark.parametrize("seqlen,causal,d,dtype", [
+    ((128, 384, 256), False, 64, "fp16"),
+    ((512, 128, 256, 128), True, 128, "bf16"),
+    ((128, 640), True, 128, "fp16"),
+])
+def test_unequal_rank_lengths(oracle, seqlen, causal, d, dtype):
+    # per-PE seqlen[] of the reference (csrc/ring_attention.cu:753): ranks of different length
+    S, P = sum(seqlen), len(seqlen)
+    w = Workload("ragged_ranks", 2, 2, d, 1, S, dtype, 71, causal)   # only used for the seeded inputs
+    q, k, v = api.make_qkv_bits(w)
+    qd, kd, vd = (to_dev(x, dtype) for x in (q, k, v))
+    plan = api.RingAttention(P, list(seqlen), d, w.batch, w.heads, dtype, causal)
+    out, lse = plan.forward(qd, kd, vd)
+    torch.cuda.synchronize()
+    rows = np.arange(w.rows)
+    check_rows(oracle, w, q, k, v, out, lse, rows)
+    # the per-step partials follow the ring schedule of the unequal chunks
+    _, _, po, pl = oracle.ring_rows(q, k, v, dtype, list(seqlen), rows, causal=causal, tile=32, want_parts=True)
+    for s in range(P):
+        o_part, lse_part = plan.block_forward(s, qd, kd, vd)
+        torch.cuda.synchronize()
+        lg = lse_part.reshape(-1).double().cpu().numpy()
+        active = np.isfinite(pl[:, s])
+        assert np.array_equal(np.isfinite(lg), active)
+        # fp32 partial; p is rounded to the storage type before the PV product (2^-9 relative for bf16)
+        assert np.abs(o_part.reshape(-1, d).double().cpu().numpy()[active] - po[active, s]).max() <= 5e-3
+    # the reference-shaped entry on the same unequal layout, one head
+    q1, k1, v1 = (np.ascontiguousarray(x[0, 0]) for x in (q, k, v))
+    o_ref, _ = oracle.attention_rows(q1[None, None], k1[None, None], v1[None, None], dtype, causal=causal)
+    start = np.concatenate([[0], np.cumsum(seqlen)])
+    for mype in range(P):
+        sl = slice(start[mype], start[mype + 1])
+        o1 = torch.empty((seqlen[mype], d), dtype=qd.dtype, device="cuda")
+        api.ring_attention(to_dev(np.ascontiguousarray(q1[sl]), dtype), to_dev(k1, dtype), to_dev(v1, dtype), o1, P, mype,
+                           list(seqlen), d, max(seqlen), causal=causal)
+        assert np.abs(o1.double().cpu().numpy() - o_ref[sl]).max() <= O_TOL
+    plan.close()
+
+
 def test_explicit_softmax_scale(oracle):
     w = Workload("scale", 1, 2, 64, 2, 256, "fp16", 31, False)
     q, k, v = api.make_qkv_bits(w)
