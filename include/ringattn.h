@@ -31,7 +31,7 @@ extern "C" {
 #define RINGATTN_ERR_DIM 3         /* dim not in {64, 128} */
 #define RINGATTN_ERR_DTYPE 4       /* dtype not fp16 / bf16 */
 #define RINGATTN_ERR_SEQLEN 5      /* a per-rank length is not a positive multiple of 128, or max_seq is below it */
-#define RINGATTN_ERR_SHAPE 6       /* batch or heads < 1, sizes overflow */
+#define RINGATTN_ERR_SHAPE 6       /* batch or heads < 1, kv_heads does not divide heads, sizes overflow */
 #define RINGATTN_ERR_WORKSPACE 7   /* caller workspace missing or too small */
 #define RINGATTN_ERR_RANK 8        /* mype / step outside [0, npes) */
 #define RINGATTN_ERR_PLAN 9        /* plan handle invalid or already destroyed */
@@ -66,6 +66,9 @@ typedef struct ringattn_params {
   int dtype;             /* RINGATTN_DTYPE_* of Q, K, V and O */
   int causal;            /* 0: every rank sees every chunk; 1: chunks in sequence order, KV chunk j > r skipped, j == r masked */
   int flags;             /* RINGATTN_FLAG_* */
+  int kv_heads;          /* heads of K and V (grouped-query attention): 0 or `heads` = one KV head per
+                            query head; otherwise it must divide `heads`, and query head h reads KV head
+                            h / (heads / kv_heads).  K and V are then [batch, kv_heads, S, dim]. */
 } ringattn_params;
 
 typedef struct ringattn_plan ringattn_plan;

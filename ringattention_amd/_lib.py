@@ -28,6 +28,7 @@ class RingattnParams(ctypes.Structure):
         ("dtype", ctypes.c_int),
         ("causal", ctypes.c_int),
         ("flags", ctypes.c_int),
+        ("kv_heads", ctypes.c_int),
     ]
 
 

@@ -39,10 +39,11 @@ def _check_tensor(t, name, dtype=None):
         raise ValueError(f"{name} must have dtype {dtype}")
 
 
-def make_params(npes, seqlen, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, flags=0):
+def make_params(npes, seqlen, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, flags=0,
+                kv_heads=0):
     arr = (ctypes.c_int * len(seqlen))(*[int(x) for x in seqlen])
     p = RingattnParams(int(npes), ctypes.cast(arr, _lib.c_int_p), int(dim), float(softmax_scale), int(batch),
-                       int(heads), DTYPE_CODE[dtype], int(bool(causal)), int(flags))
+                       int(heads), DTYPE_CODE[dtype], int(bool(causal)), int(flags), int(kv_heads))
     p._keepalive = arr
     return p
 
@@ -50,9 +51,11 @@ def make_params(npes, seqlen, dim, batch=1, heads=1, dtype="fp16", causal=False,
 class RingAttention:
     """A forward plan for P virtual ring ranks on one GPU."""
 
-    def __init__(self, npes, chunk, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, graph=False):
+    def __init__(self, npes, chunk, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, graph=False,
+                 kv_heads=0):
         """`chunk`: tokens per rank -- one int for equal chunks or a list of npes lengths
-        (the per-PE seqlen[] of csrc/ring_attention.cu:753)."""
+        (the per-PE seqlen[] of csrc/ring_attention.cu:753).  `kv_heads`: heads of K and V for
+        grouped-query attention (0 = same as `heads`)."""
         self.lib = _lib.load()
         self.seqlen = [int(chunk)] * npes if isinstance(chunk, int) else [int(x) for x in chunk]
         if len(self.seqlen) != npes:
@@ -62,8 +65,9 @@ class RingAttention:
         self.torch_dtype = TORCH_DTYPE[self.dtype_code]
         self.causal = bool(causal)
         self.seq = sum(self.seqlen)
+        self.kv_heads = kv_heads if kv_heads else heads
         self.params = make_params(npes, self.seqlen, dim, batch, heads, dtype, causal, softmax_scale,
-                                  FLAG_GRAPH if graph else 0)
+                                  FLAG_GRAPH if graph else 0, kv_heads)
         self.handle = ctypes.c_void_p()
         check(self.lib.ringattn_plan_create(ctypes.byref(self.params), None, 0, ctypes.byref(self.handle)),
               "ringattn_plan_create")
@@ -83,10 +87,11 @@ class RingAttention:
         return (self.batch, self.heads, self.seq, self.dim)
 
     def forward(self, q, k, v, out=None, lse=None, stream=None):
-        for t, nm in ((q, "q"), (k, "k"), (v, "v")):
+        kv_shape = (self.batch, self.kv_heads, self.seq, self.dim)
+        for t, nm, shp in ((q, "q", self._shape()), (k, "k", kv_shape), (v, "v", kv_shape)):
             _check_tensor(t, nm, self.torch_dtype)
-            if tuple(t.shape) != self._shape():
-                raise ValueError(f"{nm} must have shape {self._shape()}")
+            if tuple(t.shape) != shp:
+                raise ValueError(f"{nm} must have shape {shp}")
         if out is None:
             out = torch.empty_like(q)
         if lse is None:

@@ -51,6 +51,7 @@ int validate(const ringattn_params* p, Derived* d) {
   if (p->dim != 64 && p->dim != 128) return RINGATTN_ERR_DIM;
   if (p->dtype != RINGATTN_DTYPE_FP16 && p->dtype != RINGATTN_DTYPE_BF16) return RINGATTN_ERR_DTYPE;
   if (p->batch < 1 || p->heads < 1) return RINGATTN_ERR_SHAPE;
+  if (p->kv_heads < 0 || (p->kv_heads > 0 && p->heads % p->kv_heads != 0)) return RINGATTN_ERR_SHAPE;
   int64_t S = 0;
   int max_len = 0;
   for (int r = 0; r < p->npes; ++r) {
@@ -143,6 +144,8 @@ void fill_geometry(ringattn::BlockStepArgs& a, const ringattn_params& p, const D
   a.q_tiles_max = d.max_len / ringattn::kBlockM;
   a.P = p.npes;
   a.BH = (int)d.BH;
+  a.heads = p.heads;
+  a.kv_group = p.kv_heads > 0 ? p.heads / p.kv_heads : 1;
   a.causal = p.causal ? 1 : 0;
   a.scale_log2 = d.scale * 1.4426950408889634f;
   for (int r = 0; r <= p.npes; ++r) a.rank_start[r] = d.start[r];

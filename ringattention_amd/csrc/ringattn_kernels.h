@@ -19,8 +19,8 @@ constexpr int kMaxRanks = 64;
 //                      + s * part_stride_rows rows.
 struct BlockStepArgs {
   const void* q;       // [BH, S, D] storage dtype
-  const void* k;       // [BH, S, D]
-  const void* v;       // [BH, S, D]
+  const void* k;       // [batch * heads / kv_group, S, D]
+  const void* v;       // [batch * heads / kv_group, S, D]
   float* o_part;       // [BH, S, D] fp32 partial O of this step (normalised)
   float* lse_part;     // [BH, S]    fp32 partial LSE of this step (natural log)
   int64_t bh_stride;   // elements between heads (= S * D)
@@ -33,6 +33,8 @@ struct BlockStepArgs {
   int rank_base;       // first active rank of this step (pairs == nullptr)
   int n_active;        // active ranks of the step, or number of pairs
   int BH;              // batch * heads
+  int heads;           // query heads per batch entry
+  int kv_group;        // query heads per KV head (1 = one KV head per query head)
   int causal;          // chunk-level causal ring: j<r full, j==r diagonal mask
   float scale_log2;    // softmax_scale * log2(e)
   // rank r owns rows [rank_start[r], rank_start[r+1]) of every head; lengths are multiples

@@ -163,9 +163,12 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   const int first_masked = diag ? (qt * BM) / BN : n_tiles;  // tiles >= this need the causal mask
 
   const int64_t head_off = (int64_t)bh * a.bh_stride;
+  // grouped-query attention: query head h of a batch entry reads KV head h / kv_group
+  const int kv_bh = (bh / a.heads) * (a.heads / a.kv_group) + (bh % a.heads) / a.kv_group;
+  const int64_t kv_head_off = (int64_t)kv_bh * a.bh_stride;
   const char* qbase = (const char*)a.q + (head_off + (int64_t)(q_start + qt * BM) * D) * 2;
-  const char* kbase = (const char*)a.k + (head_off + (int64_t)kv_start * D) * 2;
-  const char* vbase = (const char*)a.v + (head_off + (int64_t)kv_start * D) * 2;
+  const char* kbase = (const char*)a.k + (kv_head_off + (int64_t)kv_start * D) * 2;
+  const char* vbase = (const char*)a.v + (kv_head_off + (int64_t)kv_start * D) * 2;
 
   // this lane's query rows (local to the q tile): 32 QB wave + 32 qb + n
   s16x8 qf[QB][KS];

@@ -14,9 +14,9 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 OK, E_NULL, E_NPES, E_DIM, E_DTYPE, E_SEQLEN, E_SHAPE, E_WS, E_RANK, E_PLAN, E_HIP, E_ALLOC, E_ALIGN = range(13)
 
 
-def params(npes=2, seqlen=(128, 128), dim=64, batch=1, heads=1, dtype=0, causal=0, flags=0, scale=0.0):
+def params(npes=2, seqlen=(128, 128), dim=64, batch=1, heads=1, dtype=0, causal=0, flags=0, scale=0.0, kv_heads=0):
     arr = (ctypes.c_int * max(1, len(seqlen)))(*seqlen)
-    p = RingattnParams(npes, ctypes.cast(arr, _lib.c_int_p), dim, scale, batch, heads, dtype, causal, flags)
+    p = RingattnParams(npes, ctypes.cast(arr, _lib.c_int_p), dim, scale, batch, heads, dtype, causal, flags, kv_heads)
     p._keep = arr
     return p
 
@@ -71,6 +71,8 @@ def test_parameter_validation(ralib):
     assert create(params(batch=0)) == E_SHAPE
     assert create(params(heads=-1)) == E_SHAPE
     assert create(params(scale=float("nan"))) == E_SHAPE
+    assert create(params(heads=8, kv_heads=3)) == E_SHAPE     # kv_heads must divide heads
+    assert create(params(heads=8, kv_heads=-2)) == E_SHAPE
     for bad in (params(npes=0), params(dim=7), params(seqlen=(64, 64))):
         assert wb(ctypes.byref(bad)) == 0
     assert wb(None) == 0

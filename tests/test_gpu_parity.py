@@ -150,6 +150,22 @@ def test_unequal_rank_lengths(oracle, seqlen, causal, d, dtype):
     plan.close()
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_grouped_query_heads(oracle, causal):
+    # 8 query heads share 2 KV heads: the result equals plain attention with the KV heads repeated
+    B, H, HKV, P, c, d = 2, 8, 2, 4, 256, 128
+    w = Workload("gqa", B, H, d, P, c, "bf16", 81, causal)
+    q, _, _ = api.make_qkv_bits(w)
+    wkv = Workload("gqa_kv", B, HKV, d, P, c, "bf16", 82, causal)
+    _, k, v = api.make_qkv_bits(wkv)
+    plan = api.RingAttention(P, c, d, B, H, "bf16", causal, kv_heads=HKV)
+    out, lse = plan.forward(to_dev(q, "bf16"), to_dev(k, "bf16"), to_dev(v, "bf16"))
+    torch.cuda.synchronize()
+    plan.close()
+    k_rep, v_rep = (np.repeat(x, H // HKV, axis=1) for x in (k, v))
+    check_rows(oracle, w, q, k_rep, v_rep, out, lse, np.arange(w.rows))
+
+
 def test_explicit_softmax_scale(oracle):
     w = Workload("scale", 1, 2, 64, 2, 256, "fp16", 31, False)
     q, k, v = api.make_qkv_bits(w)
