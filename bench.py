@@ -32,18 +32,12 @@ def describe(w):
             f"{w.npes} virtual ranks x {w.chunk} tokens (S={w.seq}), {w.dtype}, N(0,{w.sigma_qk:g}^2) Q/K seed {w.seed}")
 
 
-def pair_counts(w):
-    """(q, k) pairs visible in each ring step's launch."""
-    P, c = w.npes, w.chunk
-    out = []
-    for s in range(P):
-        if not w.causal:
-            out.append(P * c * c)
-        elif s == 0:
-            out.append(P * c * (c + 1) // 2)
-        else:
-            out.append(s * c * c)
-    return [x * w.batch * w.heads for x in out]
+def visible_pairs(item):
+    """(q, k) pairs of one work item (q_start, q_len, kv_start, kv_len, diag_off, slot)."""
+    _, q_len, _, kv_len, diag_off, _ = item
+    if diag_off < 0:
+        return q_len * kv_len
+    return q_len * diag_off + q_len * (q_len + 1) // 2
 
 
 def main():
@@ -52,6 +46,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg4")
+    ap.add_argument("--layout", default="contiguous", choices=["contiguous", "zigzag"],
+                    help="placement of the sequence on the ranks (zigzag: load-balanced causal ring)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the cpu_baseline sample (0 = skip)")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="only run a plain device copy of MIB mebibytes a few times and exit: the known-size kernel "
@@ -79,7 +75,7 @@ def main():
 
     q, k, v = api.make_qkv_bits(w)
     qd, kd, vd = (api.bits_to_tensor(x, w.dtype) for x in (q, k, v))
-    plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=w.graph)
+    plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=w.graph, layout=args.layout)
     out = torch.empty_like(qd)
     lse = torch.empty((w.batch, w.heads, w.seq), dtype=torch.float32, device="cuda")
     stream = torch.cuda.current_stream()
@@ -95,7 +91,7 @@ def main():
     tflops = w.flops / (ms_per_step * 1e-3) / 1e12
 
     # ---- per-kernel pass: events on the launch stream around each block launch and the merge
-    eager = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=False)
+    eager = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=False, layout=args.layout)
     o_parts = torch.empty((w.npes, w.batch, w.heads, w.seq, w.dim), dtype=torch.float32, device="cuda")
     l_parts = torch.empty((w.npes, w.batch, w.heads, w.seq), dtype=torch.float32, device="cuda")
     reps = max(3, min(args.steps, 10))
@@ -113,23 +109,22 @@ def main():
     torch.cuda.synchronize()
     block_ms = [np.mean([ev[r][s].elapsed_time(ev[r][s + 1]) for r in range(reps)]) for s in range(w.npes)]
     merge_ms = float(np.mean([ev[r][w.npes].elapsed_time(ev[r][w.npes + 1]) for r in range(reps)]))
-    pairs = pair_counts(w)
-    launch_flops = [4.0 * w.dim * p for p in pairs]
+    bh = w.batch * w.heads
+    launch_flops = [4.0 * w.dim * bh * sum(visible_pairs(it) for it in eager.work_items(s)) for s in range(w.npes)]
+    assert abs(sum(launch_flops) - w.flops) <= 1e-9 * w.flops
     block_tflops = sum(launch_flops) / (sum(block_ms) * 1e-3) / 1e12
     peak = PEAK_TFLOPS[w.dtype]
     roofline = {
         "kernel": "block_attention_kernel", "bound": "mfma",
         "achieved": round(block_tflops, 2), "peak": peak, "unit": "TFLOP/s", "frac": round(block_tflops / peak, 4),
-        "traffic": MEASURED_TRAFFIC.get(w.name),
+        "traffic": MEASURED_TRAFFIC.get(w.name) if args.layout == "contiguous" else None,
         "launches_per_step": w.npes, "avg_launch_ms": round(float(np.mean(block_ms)), 4),
         "avg_launch_flop": float(np.mean(launch_flops)),
         "per_step_ms": [round(float(x), 4) for x in block_ms],
         "per_step_tflops": [round(f / (t * 1e-3) / 1e12, 1) for f, t in zip(launch_flops, block_ms)],
     }
     # merge: algorithmic bytes = active parts * (4 d + 4) read + (2 d + 4) written, per row
-    P = w.npes
-    parts_per_rank = [(r + 1) if w.causal else P for r in range(P)]
-    merge_bytes = w.batch * w.heads * w.chunk * sum(n * (4 * w.dim + 4) + 2 * w.dim + 4 for n in parts_per_rank)
+    merge_bytes = bh * sum(ln * (bin(act).count("1") * (4 * w.dim + 4) + 2 * w.dim + 4) for _, ln, act in eager.merge_regions())
     merge = {"kernel": "merge_kernel", "bound": "hbm", "achieved": round(merge_bytes / (merge_ms * 1e-3) / 1e9, 1),
              "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(merge_bytes / (merge_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
              "ms": round(merge_ms, 4), "bytes": merge_bytes}
@@ -162,7 +157,7 @@ def main():
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w.dtype, "data": "synthetic",
-        "config": {"workload": describe(w), "algorithmic_flop": w.flops, "graph": bool(w.graph)},
+        "config": {"workload": describe(w), "algorithmic_flop": w.flops, "graph": bool(w.graph), "layout": args.layout},
         "pct_mfma_peak": round(100.0 * tflops / peak, 2),
         "roofline": roofline, "merge": merge, "cpu_baseline": cpu,
     }))

@@ -30,8 +30,8 @@ extern "C" {
 #define RINGATTN_ERR_NPES 2        /* npes < 1 or above RINGATTN_MAX_NPES */
 #define RINGATTN_ERR_DIM 3         /* dim not in {64, 128} */
 #define RINGATTN_ERR_DTYPE 4       /* dtype not fp16 / bf16 */
-#define RINGATTN_ERR_SEQLEN 5      /* a per-rank length is not a positive multiple of 128, or max_seq is below it */
-#define RINGATTN_ERR_SHAPE 6       /* batch or heads < 1, kv_heads does not divide heads, sizes overflow */
+#define RINGATTN_ERR_SEQLEN 5      /* a per-rank length is not a positive multiple of 128 (256 with the zigzag layout), or max_seq is below it */
+#define RINGATTN_ERR_SHAPE 6       /* batch or heads < 1, kv_heads does not divide heads, unknown layout, sizes overflow */
 #define RINGATTN_ERR_WORKSPACE 7   /* caller workspace missing or too small */
 #define RINGATTN_ERR_RANK 8        /* mype / step outside [0, npes) */
 #define RINGATTN_ERR_PLAN 9        /* plan handle invalid or already destroyed */
@@ -46,6 +46,18 @@ extern "C" {
 #define RINGATTN_TILE 128          /* per-rank lengths must be multiples of this; they may differ between ranks */
 
 #define RINGATTN_FLAG_GRAPH 1      /* capture the step loop + merge in a hipGraph and replay it */
+
+/*
+ * Placement of the sequence on the ranks.  CONTIGUOUS: rank r holds the tokens that follow
+ * those of rank r-1 (the reference's split, csrc/ring_attention.cu:753-757).  ZIGZAG: rank r
+ * holds two half-chunks back to back, a low one and a high one; in the sequence the low
+ * halves of ranks 0..npes-1 come first and then the high halves of ranks npes-1..0, so that
+ * under the causal mask every rank has the same amount of work (with CONTIGUOUS rank r has
+ * r + 1 visible chunks).  The reference has no causal mask and therefore no such layout; it
+ * only matters when `causal` is set.  Per-rank lengths must then be multiples of 256.
+ */
+#define RINGATTN_LAYOUT_CONTIGUOUS 0
+#define RINGATTN_LAYOUT_ZIGZAG 1
 
 /*
  * Replaces struct Ring_fwd_params (csrc/ring.h:5-19).  npes, h_seqlen, dim and
@@ -69,6 +81,7 @@ typedef struct ringattn_params {
   int kv_heads;          /* heads of K and V (grouped-query attention): 0 or `heads` = one KV head per
                             query head; otherwise it must divide `heads`, and query head h reads KV head
                             h / (heads / kv_heads).  K and V are then [batch, kv_heads, S, dim]. */
+  int layout;            /* RINGATTN_LAYOUT_*: which tokens of the sequence the rows of rank r are */
 } ringattn_params;
 
 typedef struct ringattn_plan ringattn_plan;
@@ -92,8 +105,9 @@ int ringattn_plan_destroy(ringattn_plan* plan);
 
 /*
  * The whole forward for all npes virtual ranks: replaces ring_attention()
- * (csrc/ring_attention.cu:706-722) run on every PE.  Step loop (one block-attention
- * launch per ring step, all active ranks batched) followed by one npes-way merge.
+ * (csrc/ring_attention.cu:706-722) run on every PE.  Every ring step of every rank (a few
+ * block-attention launches that each hold all steps of some ranks), then the merge of each
+ * rank's per-step partials, overlapped with the next launch on an internal stream.
  *   q, k, v : [batch, heads, S, dim] dtype     out : same shape and dtype
  *   lse     : [batch, heads, S] fp32, natural log (the reference never writes it)
  * Asynchronous on `stream` (a hipStream_t, or NULL for the default stream); the
@@ -107,8 +121,9 @@ int ringattn_fwd(ringattn_plan* plan, const void* q, const void* k, const void* 
  * One ring step (the body of the reference's step loop, csrc/ring_attention.cu:456-620,
  * for every active rank at once): rank r attends KV chunk (r + step) mod npes and the
  * normalised fp32 partial O [batch, heads, S, dim] and fp32 partial LSE
- * [batch, heads, S] are written for the rows of the active ranks.  Rows of ranks that
- * are inactive in this step (causal, chunk j > r) are left untouched.
+ * [batch, heads, S] are written for the rows of the active ranks.  Rows that see no key of
+ * the visited chunk (causal: chunk j > r; zigzag: also the low half against j > r) are
+ * left untouched.
  */
 int ringattn_block_fwd(ringattn_plan* plan, int step, const void* q, const void* k, const void* v,
                        float* o_part, float* lse_part, void* stream);
@@ -126,13 +141,37 @@ int ringattn_merge(const float* o_parts, const float* lse_parts, int n_parts, in
 /*
  * The merge as ringattn_fwd runs it, on caller-held partials: o_parts
  * [npes, batch*heads*S, dim] and lse_parts [npes, batch*heads*S] as written by
- * ringattn_block_fwd for steps 0..npes-1.  With a causal plan, part s of a row of rank r
- * is read only if rank r was active in step s (s == 0 or r + s >= npes), so parts the
- * step loop never wrote are never touched.  Like ringattn_merge, it has no counterpart
+ * ringattn_block_fwd for steps 0..npes-1.  With a causal plan, part s of a row is read
+ * only if ringattn_block_fwd writes that row in step s (contiguous layout: s == 0 or
+ * r + s >= npes for a row of rank r), so parts the step loop never wrote are never touched.  Like ringattn_merge, it has no counterpart
  * function in the reference (csrc/ring_attention.cu:207-245,621-633 pin the algebra).
  */
 int ringattn_merge_ring(ringattn_plan* plan, const float* o_parts, const float* lse_parts,
                         void* out, float* lse, void* stream);
+
+/*
+ * The schedule of a plan, for inspection (host data, no GPU work; the reference has no
+ * counterpart: its schedule is the loop `for step in 0..npes-1: kv_pe = (mype + step) % npes`
+ * of csrc/ring_attention.cu:456-470,615).  A work item is one block-attention job: the
+ * queries [q_start, q_start + q_len) of every head against the keys [kv_start, kv_start +
+ * kv_len), rows counted within a head.  diag_off < 0: every key visible; otherwise key kl
+ * (local to the KV range) is visible to query ql (local to the query range) iff
+ * kl <= ql + diag_off.  The partial result goes to slot `slot` (= the ring step).
+ * step in [0, npes): the items ringattn_block_fwd(step) runs; step == -1: all items of
+ * ringattn_fwd in launch order.  Writes min(n, capacity) items and stores n in *n_out.
+ */
+typedef struct ringattn_work_item {
+  int q_start, q_len, kv_start, kv_len, diag_off, slot;
+} ringattn_work_item;
+
+int ringattn_plan_work_items(const ringattn_plan* plan, int step, ringattn_work_item* out, int capacity, int* n_out);
+
+/*
+ * The row ranges ringattn_merge_ring merges separately: rows [start[i], start[i] + len[i])
+ * of every head read the partial slots whose bit is set in active[i].  Writes
+ * min(n, capacity) entries and stores n in *n_out.
+ */
+int ringattn_plan_merge_regions(const ringattn_plan* plan, int* start, int* len, uint64_t* active, int capacity, int* n_out);
 
 /*
  * Reference-shaped convenience entry: the signature of

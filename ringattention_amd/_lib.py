@@ -29,7 +29,13 @@ class RingattnParams(ctypes.Structure):
         ("causal", ctypes.c_int),
         ("flags", ctypes.c_int),
         ("kv_heads", ctypes.c_int),
+        ("layout", ctypes.c_int),
     ]
+
+
+class RingattnWorkItem(ctypes.Structure):
+    """struct ringattn_work_item."""
+    _fields_ = [(n, ctypes.c_int) for n in ("q_start", "q_len", "kv_start", "kv_len", "diag_off", "slot")]
 
 
 SYMBOLS = {
@@ -42,6 +48,10 @@ SYMBOLS = {
     "ringattn_merge": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
                                       ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
     "ringattn_merge_ring": (ctypes.c_int, [ctypes.c_void_p] * 6),
+    "ringattn_plan_work_items": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(RingattnWorkItem),
+                                                ctypes.c_int, c_int_p]),
+    "ringattn_plan_merge_regions": (ctypes.c_int, [ctypes.c_void_p, c_int_p, c_int_p,
+                                                   ctypes.POINTER(ctypes.c_uint64), ctypes.c_int, c_int_p]),
     "ringattn_ring_attention": (ctypes.c_int, [ctypes.c_void_p] * 5 + [ctypes.c_int, ctypes.c_int, c_int_p,
                                                                        ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                                        ctypes.c_int, ctypes.c_float]),

@@ -17,6 +17,7 @@ from ._lib import RingattnParams, check
 DTYPE_CODE = {"fp16": 0, "bf16": 1, torch.float16: 0, torch.bfloat16: 1}
 TORCH_DTYPE = {0: torch.float16, 1: torch.bfloat16}
 FLAG_GRAPH = 1
+LAYOUT_CODE = {"contiguous": 0, "zigzag": 1}
 
 
 def _stream_ptr(stream=None):
@@ -40,10 +41,10 @@ def _check_tensor(t, name, dtype=None):
 
 
 def make_params(npes, seqlen, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, flags=0,
-                kv_heads=0):
+                kv_heads=0, layout=0):
     arr = (ctypes.c_int * len(seqlen))(*[int(x) for x in seqlen])
     p = RingattnParams(int(npes), ctypes.cast(arr, _lib.c_int_p), int(dim), float(softmax_scale), int(batch),
-                       int(heads), DTYPE_CODE[dtype], int(bool(causal)), int(flags), int(kv_heads))
+                       int(heads), DTYPE_CODE[dtype], int(bool(causal)), int(flags), int(kv_heads), int(layout))
     p._keepalive = arr
     return p
 
@@ -52,10 +53,12 @@ class RingAttention:
     """A forward plan for P virtual ring ranks on one GPU."""
 
     def __init__(self, npes, chunk, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, graph=False,
-                 kv_heads=0):
+                 kv_heads=0, layout="contiguous"):
         """`chunk`: tokens per rank -- one int for equal chunks or a list of npes lengths
         (the per-PE seqlen[] of csrc/ring_attention.cu:753).  `kv_heads`: heads of K and V for
-        grouped-query attention (0 = same as `heads`)."""
+        grouped-query attention (0 = same as `heads`).  `layout`: "contiguous" (rank r holds
+        the tokens after those of rank r-1) or "zigzag" (rank r holds a low and a high
+        half-chunk; see zigzag_order)."""
         self.lib = _lib.load()
         self.seqlen = [int(chunk)] * npes if isinstance(chunk, int) else [int(x) for x in chunk]
         if len(self.seqlen) != npes:
@@ -67,7 +70,7 @@ class RingAttention:
         self.seq = sum(self.seqlen)
         self.kv_heads = kv_heads if kv_heads else heads
         self.params = make_params(npes, self.seqlen, dim, batch, heads, dtype, causal, softmax_scale,
-                                  FLAG_GRAPH if graph else 0, kv_heads)
+                                  FLAG_GRAPH if graph else 0, kv_heads, LAYOUT_CODE[layout])
         self.handle = ctypes.c_void_p()
         check(self.lib.ringattn_plan_create(ctypes.byref(self.params), None, 0, ctypes.byref(self.handle)),
               "ringattn_plan_create")
@@ -113,6 +116,24 @@ class RingAttention:
                                           _ptr(lse_part), _stream_ptr(stream)), "ringattn_block_fwd")
         return o_part, lse_part
 
+    def work_items(self, step=-1):
+        """The plan's block-attention jobs as (q_start, q_len, kv_start, kv_len, diag_off, slot)
+        tuples: those of ring step `step`, or of the whole forward in launch order (step -1)."""
+        n = ctypes.c_int()
+        check(self.lib.ringattn_plan_work_items(self.handle, int(step), None, 0, ctypes.byref(n)), "ringattn_plan_work_items")
+        items = (_lib.RingattnWorkItem * max(1, n.value))()
+        check(self.lib.ringattn_plan_work_items(self.handle, int(step), items, n.value, ctypes.byref(n)),
+              "ringattn_plan_work_items")
+        return [(w.q_start, w.q_len, w.kv_start, w.kv_len, w.diag_off, w.slot) for w in items[:n.value]]
+
+    def merge_regions(self):
+        """(start, len, active-slot bitmask) of the row ranges the ring merge handles separately."""
+        cap = 4 * self.npes
+        st, ln, act = (ctypes.c_int * cap)(), (ctypes.c_int * cap)(), (ctypes.c_uint64 * cap)()
+        n = ctypes.c_int()
+        check(self.lib.ringattn_plan_merge_regions(self.handle, st, ln, act, cap, ctypes.byref(n)),
+              "ringattn_plan_merge_regions")
+        return [(st[i], ln[i], act[i]) for i in range(n.value)]
 
     def merge_ring(self, o_parts, lse_parts, out=None, lse=None, stream=None):
         """Ring-aware merge of caller-held per-step partials [npes, B, H, S, d] / [npes, B, H, S]."""
@@ -125,6 +146,24 @@ class RingAttention:
         check(self.lib.ringattn_merge_ring(self.handle, _ptr(o_parts), _ptr(lse_parts), _ptr(out), _ptr(lse),
                                            _stream_ptr(stream)), "ringattn_merge_ring")
         return out, lse
+
+
+def zigzag_order(seqlen):
+    """Row permutation of the zigzag layout: element i is the sequence position of memory row i.
+
+    Rank r (seqlen[r] rows, back to back in memory) holds a low and a high half.  In the
+    sequence the low halves of ranks 0..P-1 come first, then the high halves of ranks P-1..0.
+    `x_memory = x_sequence[zigzag_order(seqlen)]`; invert with numpy.argsort.
+    """
+    half = [int(c) // 2 for c in seqlen]
+    P = len(half)
+    low_pos = np.concatenate(([0], np.cumsum(half)))              # start of rank r's low half
+    high_pos = low_pos[P] + np.concatenate(([0], np.cumsum(half[::-1])))  # start of the i-th high half (rank P-1-i)
+    rows = []
+    for r in range(P):
+        rows.append(np.arange(low_pos[r], low_pos[r] + half[r]))
+        rows.append(np.arange(high_pos[P - 1 - r], high_pos[P - 1 - r] + half[r]))
+    return np.concatenate(rows).astype(np.int64)
 
 
 def merge(o_parts, lse_parts, dtype, stream=None):

@@ -32,11 +32,16 @@ inline int hip_fail(hipError_t e) {
     if (e__ != hipSuccess) return hip_fail(e__); \
   } while (0)
 
+constexpr int kMaxGroups = 8;  // block launches per forward
+constexpr float kLog2e = 1.4426950408889634f;
+
 struct Derived {
   int start[RINGATTN_MAX_NPES + 1] = {};  // rank r owns rows [start[r], start[r+1]) of every head
   int max_len = 0;
+  bool zigzag = false;  // causal ring over the zigzag layout (without the mask the layouts coincide)
   int64_t S = 0;
   int64_t BH = 0;
+  int64_t kv_BH = 0;
   int64_t rows = 0;  // BH * S
   float scale = 0.f;
 };
@@ -52,25 +57,29 @@ int validate(const ringattn_params* p, Derived* d) {
   if (p->dtype != RINGATTN_DTYPE_FP16 && p->dtype != RINGATTN_DTYPE_BF16) return RINGATTN_ERR_DTYPE;
   if (p->batch < 1 || p->heads < 1) return RINGATTN_ERR_SHAPE;
   if (p->kv_heads < 0 || (p->kv_heads > 0 && p->heads % p->kv_heads != 0)) return RINGATTN_ERR_SHAPE;
+  if (p->layout != RINGATTN_LAYOUT_CONTIGUOUS && p->layout != RINGATTN_LAYOUT_ZIGZAG) return RINGATTN_ERR_SHAPE;
+  const int tile = p->layout == RINGATTN_LAYOUT_ZIGZAG ? 2 * RINGATTN_TILE : RINGATTN_TILE;
   int64_t S = 0;
   int max_len = 0;
   for (int r = 0; r < p->npes; ++r) {
     const int c = p->h_seqlen[r];
-    if (c <= 0 || c % RINGATTN_TILE != 0) return RINGATTN_ERR_SEQLEN;
+    if (c <= 0 || c % tile != 0) return RINGATTN_ERR_SEQLEN;
     S += c;
     if (c > max_len) max_len = c;
   }
   const int64_t BH = (int64_t)p->batch * p->heads;
   if (S > INT32_MAX / 2 || BH > INT32_MAX / 2) return RINGATTN_ERR_SHAPE;
-  if (BH * p->npes > (int64_t)INT32_MAX / 64) return RINGATTN_ERR_SHAPE;  // grid size
+  if (BH * p->npes * p->npes > (int64_t)INT32_MAX / 64) return RINGATTN_ERR_SHAPE;  // grid size
   if (BH * S > (int64_t)1 << 40) return RINGATTN_ERR_SHAPE;
   if (!std::isfinite(p->softmax_scale)) return RINGATTN_ERR_SHAPE;
   if (d) {
     d->start[0] = 0;
     for (int r = 0; r < p->npes; ++r) d->start[r + 1] = d->start[r] + p->h_seqlen[r];
     d->max_len = max_len;
+    d->zigzag = p->layout == RINGATTN_LAYOUT_ZIGZAG && p->causal;
     d->S = S;
     d->BH = BH;
+    d->kv_BH = p->kv_heads > 0 ? (int64_t)p->batch * p->kv_heads : BH;
     d->rows = BH * S;
     d->scale = p->softmax_scale > 0.f ? p->softmax_scale : 1.0f / std::sqrt((float)p->dim);
   }
@@ -79,18 +88,60 @@ int validate(const ringattn_params* p, Derived* d) {
 
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
-constexpr int kMaxGroups = 8;  // launches per forward
-
 size_t workspace_bytes_of(const ringattn_params* p, const Derived& d) {
   return (size_t)p->npes * (size_t)d.rows * (size_t)(p->dim + 1) * sizeof(float);
 }
 
+inline ringattn::WorkItem make_item(int q_start, int q_len, int kv_start, int kv_len, int diag_off, int slot) {
+  ringattn::WorkItem w;
+  w.q_start = q_start;
+  w.q_len = q_len;
+  w.kv_start = kv_start;
+  w.kv_len = kv_len;
+  w.diag_off = diag_off;
+  w.slot = slot;
+  w.pad0 = w.pad1 = 0;
+  return w;
+}
+
+// The work of virtual rank r at ring step s: it visits the KV of rank j = (r + s) mod P
+// (csrc/ring_attention.cu:463,531,615).  Partials go to slot s.
+//   no mask            : all queries of r against all keys of j;
+//   causal, contiguous : j > r nothing, j == r diagonal, j < r everything;
+//   causal, zigzag     : rank r holds a low half (sequence position r) and a high half
+//       (position 2P-1-r) back to back.  The low queries see the low keys of j <= r; the high
+//       queries see every low half and the high halves of j >= r.  So: j < r, all queries of
+//       r against the low half of j; j == r, the plain diagonal over the whole chunk (its
+//       low half precedes its high half in the sequence too); j > r, the high queries of r
+//       against the whole chunk of j.  Every rank does the same amount of work.
+void append_items(std::vector<ringattn::WorkItem>& out, const Derived& d, int P, bool causal, int r, int s) {
+  const int j = (r + s) % P;
+  const int q0 = d.start[r], ql = d.start[r + 1] - q0;
+  const int k0 = d.start[j], kl = d.start[j + 1] - k0;
+  if (!causal) {
+    out.push_back(make_item(q0, ql, k0, kl, -1, s));
+  } else if (j == r) {
+    out.push_back(make_item(q0, ql, k0, kl, 0, s));
+  } else if (!d.zigzag) {
+    if (j < r) out.push_back(make_item(q0, ql, k0, kl, -1, s));
+  } else {
+    if (j < r) out.push_back(make_item(q0, ql, k0, kl / 2, -1, s));
+    else out.push_back(make_item(q0 + ql / 2, ql / 2, k0, kl, -1, s));
+  }
+}
+
 }  // namespace
 
-// One launch of the forward: the (rank, step) pairs of a few virtual ranks, all their steps.
+// One block launch of the forward: all ring steps of a few virtual ranks.
 struct LaunchGroup {
-  int pair_begin, pair_count;  // slice of the pair table
-  int rank_begin, rank_count;  // slice of group_ranks
+  int item_begin, item_count;      // slice of the item table
+  int region_begin, region_count;  // slice of `regions`: what is merged after this launch
+};
+
+// Rows [start, start + len) of every head share one set of active partial slots.
+struct MergeRegion {
+  int start, len;
+  uint64_t active;
 };
 
 struct ringattn_plan {
@@ -102,14 +153,19 @@ struct ringattn_plan {
   bool own_ws = false;
   float* o_parts = nullptr;    // [npes, rows, dim]
   float* lse_parts = nullptr;  // [npes, rows]
-  // Launch schedule of ringattn_fwd.  The ring steps of different ranks are independent
-  // (each (rank, step) pair writes its own rows of its step's partial slot), so the forward
-  // is issued as a few launches that each hold ALL steps of a few ranks; the merge of those
-  // ranks then runs on a second stream underneath the next launch.
-  std::vector<int> h_pairs;       // packed (rank << 16 | step), launch by launch
-  std::vector<int> group_ranks;
+  // Item table (host copy + device copy made at the first forward): first the launch
+  // schedule of ringattn_fwd, then one list per ring step for ringattn_block_fwd.
+  // The ring steps of different ranks are independent (each item writes its own rows of its
+  // step's partial slot), so the forward is issued as a few launches that each hold ALL
+  // steps of a few ranks; the merge of those ranks then runs on a second stream underneath
+  // the next launch.
+  std::vector<ringattn::WorkItem> h_items;
   std::vector<LaunchGroup> groups;
-  int* d_pairs = nullptr;         // device copy of h_pairs (allocated at the first forward)
+  std::vector<MergeRegion> regions;  // group by group, then (from all_regions on) rank by rank
+  int all_regions = 0;
+  std::vector<int> step_begin;       // [npes + 1] slices of h_items, one per ring step
+  int q_tiles_max = 0;
+  ringattn::WorkItem* d_items = nullptr;
   hipStream_t merge_stream = nullptr;
   hipEvent_t ev_group[kMaxGroups]{};
   hipEvent_t ev_done = nullptr;
@@ -125,115 +181,103 @@ struct ringattn_plan {
 
 namespace {
 
-// Active ranks of ring step s.  Non-causal: all.  Causal: KV chunk j = (r + s) mod P is
-// visible iff j <= r, i.e. s == 0 (diagonal) or r + s >= P (wrapped, j < r).
-inline void active_ranks(int P, int causal, int s, int* rank_base, int* n_active) {
-  if (!causal || s == 0) {
-    *rank_base = 0;
-    *n_active = P;
-  } else {
-    *rank_base = P - s;
-    *n_active = s;
-  }
-}
-
 // fields of the launch arguments that depend only on the geometry
 void fill_geometry(ringattn::BlockStepArgs& a, const ringattn_params& p, const Derived& d) {
   a.bh_stride = d.S * p.dim;
+  a.kv_bh_stride = d.S * p.dim;
+  a.part_stride_rows = d.rows;
   a.S = (int)d.S;
-  a.q_tiles_max = d.max_len / ringattn::kBlockM;
-  a.P = p.npes;
+  a.slot_bias = 0;
   a.BH = (int)d.BH;
   a.heads = p.heads;
   a.kv_group = p.kv_heads > 0 ? p.heads / p.kv_heads : 1;
-  a.causal = p.causal ? 1 : 0;
-  a.scale_log2 = d.scale * 1.4426950408889634f;
-  for (int r = 0; r <= p.npes; ++r) a.rank_start[r] = d.start[r];
+  a.scale_log2 = d.scale * kLog2e;
 }
 
-int launch_step(const ringattn_plan* pl, int s, const void* q, const void* k, const void* v,
-                float* o_part, float* lse_part, hipStream_t stream) {
-  ringattn::BlockStepArgs a;
-  fill_geometry(a, pl->p, pl->d);
-  a.q = q;
-  a.k = k;
-  a.v = v;
-  a.o_part = o_part;
-  a.lse_part = lse_part;
-  a.pairs = nullptr;
-  a.part_stride_rows = 0;
-  a.step = s;
-  active_ranks(pl->p.npes, pl->p.causal, s, &a.rank_base, &a.n_active);
-  RA_HIP(ringattn::launch_block_step(a, pl->p.dtype, pl->p.dim, stream));
-  return RINGATTN_OK;
+// The rows of rank r that share a set of active slots, with that set: slot s is active for
+// a row iff the item list of (r, s) covers the row.
+void append_regions(std::vector<MergeRegion>& out, const Derived& d, int P, bool causal, int r) {
+  const int q0 = d.start[r], ql = d.start[r + 1] - q0;
+  const int parts = d.zigzag ? 2 : 1;
+  for (int i = 0; i < parts; ++i) {
+    MergeRegion m;
+    m.start = q0 + i * (ql / parts);
+    m.len = ql / parts;
+    m.active = 0;
+    std::vector<ringattn::WorkItem> items;
+    for (int s = 0; s < P; ++s) {
+      items.clear();
+      append_items(items, d, P, causal, r, s);
+      for (const auto& w : items)
+        if (w.q_start <= m.start && m.start + m.len <= w.q_start + w.q_len) m.active |= (uint64_t)1 << s;
+    }
+    out.push_back(m);
+  }
 }
 
-// merge of the rows of one virtual rank; with a causal ring, part s of rank r is active iff
-// s == 0 or r + s >= P, and inactive parts are never read
-int launch_rank_merge(const ringattn_plan* pl, const float* o_parts, const float* lse_parts, void* out,
-                      float* lse, hipStream_t stream, int rank) {
-  ringattn::MergeArgs m;
-  m.o_parts = o_parts;
-  m.lse_parts = lse_parts;
-  m.out = out;
-  m.lse = lse;
-  m.sel_start = pl->d.start[rank];
-  m.sel_len = pl->d.start[rank + 1] - pl->d.start[rank];
-  m.rows = pl->d.BH * m.sel_len;
-  m.part_stride_rows = pl->d.rows;
-  m.n_parts = pl->p.npes;
-  m.first_wrapped = pl->p.causal ? pl->p.npes - rank : 1;
-  m.S = (int)pl->d.S;
-  RA_HIP(ringattn::launch_merge(m, pl->p.dtype, pl->p.dim, stream));
-  return RINGATTN_OK;
-}
-
-// Launch schedule.  Causal: rank r has r + 1 visible chunks, so ranks are paired (P-1-g, g)
-// to give every launch the same work; non-causal: consecutive ranks.  At most kMaxGroups
-// launches.  Within a launch the pairs of one rank are listed in ring order
-// (csrc/ring_attention.cu:456-470: step s visits chunk (r + s) mod P).
+// Launch schedule.  Contiguous causal: rank r has r + 1 visible chunks, so ranks are paired
+// (P-1-g, g) to give every launch the same work; otherwise (no mask, or zigzag, where all
+// ranks have equal work) consecutive ranks.  At most kMaxGroups launches.  Within a launch
+// the items of one rank are listed in ring order.
 void build_schedule(ringattn_plan* pl) {
   const int P = pl->p.npes;
+  const Derived& d = pl->d;
   const bool causal = pl->p.causal != 0;
+  const bool paired = causal && !d.zigzag;
   std::vector<int> order;  // ranks in launch order
-  if (causal) {
+  if (paired) {
     for (int g = 0; g < (P + 1) / 2; ++g) {
       order.push_back(P - 1 - g);
       if (g != P - 1 - g) order.push_back(g);
     }
+  } else if (d.zigzag) {
+    // rank 0 merges the fewest partials: last, where the merge is not hidden under a launch
+    for (int r = P - 1; r >= 0; --r) order.push_back(r);
   } else {
     for (int r = 0; r < P; ++r) order.push_back(r);
   }
-  const int n_groups = P < 4 ? 1 : (P / 2 < kMaxGroups ? (causal ? (P + 1) / 2 : (P < 8 ? P / 2 : 4)) : (causal ? kMaxGroups : 4));
+  int n_groups;
+  if (P < 4) n_groups = 1;
+  else if (paired) n_groups = (P + 1) / 2 < kMaxGroups ? (P + 1) / 2 : kMaxGroups;
+  else n_groups = P < 8 ? P / 2 : 4;
   size_t pos = 0;
   for (int g = 0; g < n_groups; ++g) {
-    // even split of the rank list; causal lists come in balanced pairs, keep pairs together
-    size_t end = (size_t)order.size() * (g + 1) / n_groups;
-    if (causal && (end & 1) && end < order.size()) ++end;
+    // even split of the rank list; paired lists come in balanced pairs, keep pairs together
+    size_t end = order.size() * (size_t)(g + 1) / (size_t)n_groups;
+    if (paired && (end & 1) && end < order.size()) ++end;
     if (g == n_groups - 1) end = order.size();
     if (end <= pos) continue;
     LaunchGroup lg;
-    lg.pair_begin = (int)pl->h_pairs.size();
-    lg.rank_begin = (int)pl->group_ranks.size();
+    lg.item_begin = (int)pl->h_items.size();
+    lg.region_begin = (int)pl->regions.size();
     for (size_t i = pos; i < end; ++i) {
       const int r = order[i];
-      pl->group_ranks.push_back(r);
-      for (int s = 0; s < P; ++s) {
-        const int j = (r + s) % P;
-        if (!causal || j <= r) pl->h_pairs.push_back((r << 16) | s);
-      }
+      append_regions(pl->regions, d, P, causal, r);
+      for (int s = 0; s < P; ++s) append_items(pl->h_items, d, P, causal, r, s);
     }
-    lg.pair_count = (int)pl->h_pairs.size() - lg.pair_begin;
-    lg.rank_count = (int)pl->group_ranks.size() - lg.rank_begin;
+    lg.item_count = (int)pl->h_items.size() - lg.item_begin;
+    lg.region_count = (int)pl->regions.size() - lg.region_begin;
     pl->groups.push_back(lg);
     pos = end;
   }
+  pl->all_regions = (int)pl->regions.size();
+  for (int r = 0; r < P; ++r) append_regions(pl->regions, d, P, causal, r);
+  // per-step lists: one ring step of every rank
+  for (int s = 0; s < P; ++s) {
+    pl->step_begin.push_back((int)pl->h_items.size());
+    for (int r = 0; r < P; ++r) append_items(pl->h_items, d, P, causal, r, s);
+  }
+  pl->step_begin.push_back((int)pl->h_items.size());
+  int longest = 0;
+  for (const auto& w : pl->h_items) longest = w.q_len > longest ? w.q_len : longest;
+  pl->q_tiles_max = longest / ringattn::kBlockM;
 }
 
 int ensure_streams(ringattn_plan* pl) {
   if (pl->streams_ready) return RINGATTN_OK;
-  RA_HIP(hipMalloc((void**)&pl->d_pairs, pl->h_pairs.size() * sizeof(int)));
-  RA_HIP(hipMemcpy(pl->d_pairs, pl->h_pairs.data(), pl->h_pairs.size() * sizeof(int), hipMemcpyHostToDevice));
+  const size_t bytes = pl->h_items.size() * sizeof(ringattn::WorkItem);
+  RA_HIP(hipMalloc((void**)&pl->d_items, bytes));
+  RA_HIP(hipMemcpy(pl->d_items, pl->h_items.data(), bytes, hipMemcpyHostToDevice));
   RA_HIP(hipStreamCreateWithFlags(&pl->merge_stream, hipStreamNonBlocking));
   for (int i = 0; i < kMaxGroups; ++i) RA_HIP(hipEventCreateWithFlags(&pl->ev_group[i], hipEventDisableTiming));
   RA_HIP(hipEventCreateWithFlags(&pl->ev_done, hipEventDisableTiming));
@@ -241,21 +285,38 @@ int ensure_streams(ringattn_plan* pl) {
   return RINGATTN_OK;
 }
 
-int launch_group(const ringattn_plan* pl, const LaunchGroup& lg, const void* q, const void* k, const void* v,
-                 hipStream_t stream) {
+// A block launch over a slice of the item table; o_part / lse_part: partial slot `slot_bias`.
+int launch_items(const ringattn_plan* pl, int item_begin, int item_count, const void* q, const void* k,
+                 const void* v, float* o_part, float* lse_part, int slot_bias, hipStream_t stream) {
   ringattn::BlockStepArgs a;
   fill_geometry(a, pl->p, pl->d);
   a.q = q;
   a.k = k;
   a.v = v;
-  a.o_part = pl->o_parts;
-  a.lse_part = pl->lse_parts;
-  a.pairs = pl->d_pairs + lg.pair_begin;
-  a.part_stride_rows = pl->d.rows;
-  a.step = 0;
-  a.rank_base = 0;
-  a.n_active = lg.pair_count;
+  a.o_part = o_part;
+  a.lse_part = lse_part;
+  a.items = pl->d_items + item_begin;
+  a.n_items = item_count;
+  a.q_tiles_max = pl->q_tiles_max;
+  a.slot_bias = slot_bias;
   RA_HIP(ringattn::launch_block_step(a, pl->p.dtype, pl->p.dim, stream));
+  return RINGATTN_OK;
+}
+
+int launch_region_merge(const ringattn_plan* pl, const float* o_parts, const float* lse_parts, void* out,
+                        float* lse, hipStream_t stream, const MergeRegion& reg) {
+  ringattn::MergeArgs m;
+  m.o_parts = o_parts;
+  m.lse_parts = lse_parts;
+  m.out = out;
+  m.lse = lse;
+  m.sel_start = reg.start;
+  m.sel_len = reg.len;
+  m.rows = pl->d.BH * reg.len;
+  m.part_stride_rows = pl->d.rows;
+  m.active = reg.active;
+  m.S = (int)pl->d.S;
+  RA_HIP(ringattn::launch_merge(m, pl->p.dtype, pl->p.dim, stream));
   return RINGATTN_OK;
 }
 
@@ -269,7 +330,7 @@ int run_forward(ringattn_plan* pl, const void* q, const void* k, const void* v, 
   const size_t G = pl->groups.size();
   for (size_t g = 0; g < G; ++g) {
     const LaunchGroup& lg = pl->groups[g];
-    rc = launch_group(pl, lg, q, k, v, stream);
+    rc = launch_items(pl, lg.item_begin, lg.item_count, q, k, v, pl->o_parts, pl->lse_parts, 0, stream);
     if (rc != RINGATTN_OK) return rc;
     hipStream_t ms = stream;
     if (g + 1 < G) {
@@ -277,8 +338,8 @@ int run_forward(ringattn_plan* pl, const void* q, const void* k, const void* v, 
       RA_HIP(hipStreamWaitEvent(pl->merge_stream, pl->ev_group[g], 0));
       ms = pl->merge_stream;
     }
-    for (int i = 0; i < lg.rank_count; ++i) {
-      rc = launch_rank_merge(pl, pl->o_parts, pl->lse_parts, out, lse, ms, pl->group_ranks[lg.rank_begin + i]);
+    for (int i = 0; i < lg.region_count; ++i) {
+      rc = launch_region_merge(pl, pl->o_parts, pl->lse_parts, out, lse, ms, pl->regions[lg.region_begin + i]);
       if (rc != RINGATTN_OK) return rc;
     }
   }
@@ -366,7 +427,7 @@ int ringattn_plan_destroy(ringattn_plan* plan) {
     (void)hipStreamDestroy(plan->merge_stream);
     for (int i = 0; i < kMaxGroups; ++i) (void)hipEventDestroy(plan->ev_group[i]);
     (void)hipEventDestroy(plan->ev_done);
-    (void)hipFree(plan->d_pairs);
+    (void)hipFree(plan->d_items);
   }
   if (plan->own_ws && plan->ws) {
     hipError_t e = hipFree(plan->ws);
@@ -387,7 +448,7 @@ int ringattn_fwd(ringattn_plan* plan, const void* q, const void* k, const void* 
   if (rc0 != RINGATTN_OK) return rc0;
   if (!(plan->p.flags & RINGATTN_FLAG_GRAPH)) return run_forward(plan, q, k, v, out, lse, stream);
 
-  // hipGraph replay: the P + 1 launches are captured once per pointer set on a private
+  // hipGraph replay: the launches of a forward are captured once per pointer set on a private
   // stream (kernel nodes only, no memset nodes) and replayed on the caller's stream.
   if (!plan->exec || plan->gq != q || plan->gk != k || plan->gv != v || plan->gout != out || plan->glse != lse) {
     drop_graph(plan);
@@ -423,7 +484,10 @@ int ringattn_block_fwd(ringattn_plan* plan, int step, const void* q, const void*
   if (!q || !k || !v || !o_part || !lse_part) return RINGATTN_ERR_NULL;
   if (step < 0 || step >= plan->p.npes) return RINGATTN_ERR_RANK;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o_part) || ((uintptr_t)lse_part & 3u)) return RINGATTN_ERR_ALIGN;
-  return launch_step(plan, step, q, k, v, o_part, lse_part, (hipStream_t)stream);
+  int rc = ensure_streams(plan);
+  if (rc != RINGATTN_OK) return rc;
+  return launch_items(plan, plan->step_begin[step], plan->step_begin[step + 1] - plan->step_begin[step], q, k, v,
+                      o_part, lse_part, step, (hipStream_t)stream);
 }
 
 int ringattn_merge_ring(ringattn_plan* plan, const float* o_parts, const float* lse_parts, void* out,
@@ -431,9 +495,37 @@ int ringattn_merge_ring(ringattn_plan* plan, const float* o_parts, const float* 
   if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
   if (!o_parts || !lse_parts || !out || !lse) return RINGATTN_ERR_NULL;
   if (!aligned16(o_parts) || !aligned16(out) || ((uintptr_t)lse_parts & 3u) || ((uintptr_t)lse & 3u)) return RINGATTN_ERR_ALIGN;
-  for (int r = 0; r < plan->p.npes; ++r) {
-    int rc = launch_rank_merge(plan, o_parts, lse_parts, out, lse, (hipStream_t)stream, r);
+  for (size_t i = (size_t)plan->all_regions; i < plan->regions.size(); ++i) {
+    int rc = launch_region_merge(plan, o_parts, lse_parts, out, lse, (hipStream_t)stream, plan->regions[i]);
     if (rc != RINGATTN_OK) return rc;
+  }
+  return RINGATTN_OK;
+}
+
+int ringattn_plan_work_items(const ringattn_plan* plan, int step, ringattn_work_item* out, int capacity, int* n_out) {
+  if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
+  if (!n_out || (capacity > 0 && !out)) return RINGATTN_ERR_NULL;
+  if (step < -1 || step >= plan->p.npes) return RINGATTN_ERR_RANK;
+  const int begin = step < 0 ? 0 : plan->step_begin[step];
+  const int end = step < 0 ? plan->step_begin[0] : plan->step_begin[step + 1];
+  *n_out = end - begin;
+  for (int i = begin; i < end && i - begin < capacity; ++i) {
+    const ringattn::WorkItem& w = plan->h_items[i];
+    out[i - begin] = ringattn_work_item{w.q_start, w.q_len, w.kv_start, w.kv_len, w.diag_off, w.slot};
+  }
+  return RINGATTN_OK;
+}
+
+int ringattn_plan_merge_regions(const ringattn_plan* plan, int* start, int* len, uint64_t* active, int capacity, int* n_out) {
+  if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
+  if (!n_out || (capacity > 0 && (!start || !len || !active))) return RINGATTN_ERR_NULL;
+  const int n = (int)plan->regions.size() - plan->all_regions;
+  *n_out = n;
+  for (int i = 0; i < n && i < capacity; ++i) {
+    const MergeRegion& m = plan->regions[plan->all_regions + i];
+    start[i] = m.start;
+    len[i] = m.len;
+    active[i] = m.active;
   }
   return RINGATTN_OK;
 }
@@ -441,7 +533,7 @@ int ringattn_merge_ring(ringattn_plan* plan, const float* o_parts, const float* 
 int ringattn_merge(const float* o_parts, const float* lse_parts, int n_parts, int64_t rows, int dim,
                    int dtype, void* out, float* lse, void* stream) {
   if (!o_parts || !lse_parts || !out || !lse) return RINGATTN_ERR_NULL;
-  if (n_parts < 1 || n_parts > RINGATTN_MAX_NPES) return RINGATTN_ERR_NPES;
+  if (n_parts < 1 || n_parts > ringattn::kMaxParts) return RINGATTN_ERR_NPES;
   if (dim != 64 && dim != 128) return RINGATTN_ERR_DIM;
   if (dtype != RINGATTN_DTYPE_FP16 && dtype != RINGATTN_DTYPE_BF16) return RINGATTN_ERR_DTYPE;
   if (rows < 0 || rows > ((int64_t)1 << 40)) return RINGATTN_ERR_SHAPE;
@@ -453,8 +545,7 @@ int ringattn_merge(const float* o_parts, const float* lse_parts, int n_parts, in
   m.lse = lse;
   m.rows = rows;
   m.part_stride_rows = rows;
-  m.n_parts = n_parts;
-  m.first_wrapped = 1;
+  m.active = n_parts >= 64 ? ~(uint64_t)0 : (((uint64_t)1 << n_parts) - 1);
   m.S = (int)(rows > 0 ? (rows < INT32_MAX ? rows : INT32_MAX) : 1);
   m.sel_start = 0;
   m.sel_len = m.S;
@@ -483,44 +574,45 @@ int ringattn_ring_attention(const void* q, const void* k, const void* v, void* o
   if (!q || !k || !v || !out) return RINGATTN_ERR_NULL;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return RINGATTN_ERR_ALIGN;
 
-  // steps in which rank mype has a visible chunk, in ring order
-  std::vector<int> steps;
+  // the visible ring steps of rank mype in ring order, one compact partial slot each; the
+  // query rows are local to the caller's rank-sized q and out buffers
+  const int c = d.start[mype + 1] - d.start[mype];  // rows of this rank
+  std::vector<ringattn::WorkItem> items;
   for (int s = 0; s < npes; ++s) {
     const int j = (mype + s) % npes;
-    if (!causal || j <= mype) steps.push_back(s);
+    if (causal && j > mype) continue;
+    items.push_back(make_item(0, c, d.start[j], d.start[j + 1] - d.start[j], (causal && j == mype) ? 0 : -1, (int)items.size()));
   }
-  const int n_parts = (int)steps.size();
-  const size_t c = (size_t)(d.start[mype + 1] - d.start[mype]);  // rows of this rank
-  const size_t first = (size_t)d.start[mype];
+  const int n_parts = (int)items.size();
   // per-call scratch, like the reference's per-call allocations (:383-394) but freed
   float* ws = nullptr;
-  RA_HIP(hipMalloc((void**)&ws, (size_t)n_parts * c * (size_t)(dim + 1) * sizeof(float) + c * sizeof(float)));
+  const size_t table_bytes = (size_t)n_parts * sizeof(ringattn::WorkItem);
+  RA_HIP(hipMalloc((void**)&ws, (size_t)n_parts * c * (size_t)(dim + 1) * sizeof(float) + (size_t)c * sizeof(float) + table_bytes));
   float* o_parts = ws;
   float* lse_parts = ws + (size_t)n_parts * c * dim;
   float* lse_tmp = lse_parts + (size_t)n_parts * c;
-  const size_t esz = 2;
-  // The kernel addresses the rows of rank r at rank_start[r]: shift the rank-local buffers
-  // so that rank mype's rows land on them.  The shifted pointers are never dereferenced
-  // outside [start[mype], start[mype + 1]).
-  const char* q_shift = (const char*)q - first * dim * esz;
-  for (int i = 0; i < n_parts && rc == RINGATTN_OK; ++i) {
+  ringattn::WorkItem* d_items = (ringattn::WorkItem*)(lse_tmp + c);  // 16-byte aligned: c is a multiple of 128
+  hipError_t e = hipMemcpy(d_items, items.data(), table_bytes, hipMemcpyHostToDevice);
+  if (e != hipSuccess) rc = hip_fail(e);
+  if (rc == RINGATTN_OK) {
     ringattn::BlockStepArgs a;
     fill_geometry(a, p, d);
-    a.q = q_shift;
+    a.q = q;
     a.k = k;
     a.v = v;
-    a.o_part = o_parts + (size_t)i * c * dim - first * dim;
-    a.lse_part = lse_parts + (size_t)i * c - first;
-    a.pairs = nullptr;
-    a.part_stride_rows = 0;
-    a.step = steps[i];
-    a.rank_base = mype;
-    a.n_active = 1;
-    hipError_t e = ringattn::launch_block_step(a, dtype, dim, nullptr);
+    a.o_part = o_parts;
+    a.lse_part = lse_parts;
+    a.items = d_items;
+    a.n_items = n_parts;
+    a.q_tiles_max = c / ringattn::kBlockM;
+    a.bh_stride = (int64_t)c * dim;
+    a.part_stride_rows = c;
+    a.S = c;
+    e = ringattn::launch_block_step(a, dtype, dim, nullptr);
     if (e != hipSuccess) rc = hip_fail(e);
   }
   if (rc == RINGATTN_OK) rc = ringattn_merge(o_parts, lse_parts, n_parts, (int64_t)c, dim, dtype, out, lse ? lse : lse_tmp, nullptr);
-  hipError_t e = hipDeviceSynchronize();  // blocking, as csrc/ring_attention.cu:721
+  e = hipDeviceSynchronize();  // blocking, as csrc/ring_attention.cu:721
   if (rc == RINGATTN_OK && e != hipSuccess) rc = hip_fail(e);
   (void)hipFree(ws);
   return rc;
@@ -533,8 +625,8 @@ const char* ringattn_strerror(int code) {
     case RINGATTN_ERR_NPES: return "npes out of range";
     case RINGATTN_ERR_DIM: return "dim must be 64 or 128";
     case RINGATTN_ERR_DTYPE: return "dtype must be fp16 (0) or bf16 (1)";
-    case RINGATTN_ERR_SEQLEN: return "per-rank sequence lengths must be positive multiples of 128 (and max_seq at least the longest)";
-    case RINGATTN_ERR_SHAPE: return "batch/heads/scale invalid or sizes overflow";
+    case RINGATTN_ERR_SEQLEN: return "per-rank sequence lengths must be positive multiples of 128 (256 with the zigzag layout), and max_seq at least the longest";
+    case RINGATTN_ERR_SHAPE: return "batch/heads/kv_heads/layout/scale invalid or sizes overflow";
     case RINGATTN_ERR_WORKSPACE: return "workspace too small";
     case RINGATTN_ERR_RANK: return "rank or step outside [0, npes)";
     case RINGATTN_ERR_PLAN: return "invalid or destroyed plan";

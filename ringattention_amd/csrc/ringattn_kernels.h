@@ -7,53 +7,55 @@
 namespace ringattn {
 
 constexpr int kBlockM = 128;  // query rows per workgroup (4 waves x 32 rows)
-constexpr int kMaxRanks = 64;
+constexpr int kMaxParts = 64; // partial slots a merge can combine
 
-// A batch of (rank, ring step) pairs: rank r at step s works on KV chunk (r + s) mod P --
-// the launch-level restatement of the step loop body of the reference kernel
-// (csrc/ring_attention.cu:456-470,531-610).  Two ways to name the pairs:
-//   pairs == nullptr : one ring step for the ranks rank_base .. rank_base + n_active - 1;
-//                      o_part / lse_part point at that step's slot;
-//   pairs != nullptr : n_active packed pairs (rank << 16 | step) read from device memory;
-//                      o_part / lse_part point at slot 0 and step s is written at
-//                      + s * part_stride_rows rows.
+// One unit of block-attention work: the queries [q_start, q_start + q_len) of every head
+// against the keys/values [kv_start, kv_start + kv_len) of the matching KV head -- the body
+// of one ring step of one rank (csrc/ring_attention.cu:456-470,531-610: rank r at step s
+// works on the KV chunk of rank (r + s) mod P).  Row numbers are local to a head's [S, D]
+// slab; all four are multiples of kBlockM.  The normalised partial O and the partial LSE
+// of the item go to partial slot `slot`, at the rows of its queries.
+struct WorkItem {
+  int q_start, q_len;
+  int kv_start, kv_len;
+  int diag_off;  // < 0: every key is visible.  >= 0: key kl (local to the KV range) is visible
+                 // to query ql (local to the query range) iff kl <= ql + diag_off; then
+                 // diag_off + q_len <= kv_len
+  int slot;
+  int pad0, pad1;
+};
+static_assert(sizeof(WorkItem) == 32, "WorkItem is read as two 16-byte scalar loads");
+
 struct BlockStepArgs {
   const void* q;       // [BH, S, D] storage dtype
   const void* k;       // [batch * heads / kv_group, S, D]
   const void* v;       // [batch * heads / kv_group, S, D]
-  float* o_part;       // [BH, S, D] fp32 partial O of this step (normalised)
-  float* lse_part;     // [BH, S]    fp32 partial LSE of this step (natural log)
-  int64_t bh_stride;   // elements between heads (= S * D)
-  int S;               // tokens per head
-  int q_tiles_max;     // kBlockM-row q tiles of the longest rank (grid dimension)
-  int P;               // virtual ranks
-  const int* pairs;    // device array of packed (rank, step) pairs, or nullptr
-  int64_t part_stride_rows;  // rows between the partial slots of consecutive steps
-  int step;            // ring step s (pairs == nullptr)
-  int rank_base;       // first active rank of this step (pairs == nullptr)
-  int n_active;        // active ranks of the step, or number of pairs
+  float* o_part;       // partial slot `slot_bias`: [BH, S, D] fp32 partial O (normalised)
+  float* lse_part;     // partial slot `slot_bias`: [BH, S] fp32 partial LSE (natural log)
+  const WorkItem* items;     // device array
+  int64_t bh_stride;   // elements between heads of q (= S * D)
+  int64_t kv_bh_stride;      // elements between heads of k and v
+  int64_t part_stride_rows;  // rows between consecutive partial slots
+  int S;               // rows per head in the partial slots
+  int q_tiles_max;     // kBlockM-row q tiles of the longest item (grid dimension)
+  int n_items;
+  int slot_bias;       // item.slot - slot_bias is the slot index relative to o_part / lse_part
   int BH;              // batch * heads
   int heads;           // query heads per batch entry
   int kv_group;        // query heads per KV head (1 = one KV head per query head)
-  int causal;          // chunk-level causal ring: j<r full, j==r diagonal mask
   float scale_log2;    // softmax_scale * log2(e)
-  // rank r owns rows [rank_start[r], rank_start[r+1]) of every head; lengths are multiples
-  // of kBlockM and may differ per rank (the per-PE seqlen[] of csrc/ring_attention.cu:753)
-  int rank_start[kMaxRanks + 1];
 };
 
-// n-way merge of (O, LSE) partials into the final O (storage dtype) and LSE, for the rows
-// [sel_start, sel_start + sel_len) of every head (one virtual rank, or everything).
+// Merge of (O, LSE) partials into the final O (storage dtype) and LSE, for the rows
+// [sel_start, sel_start + sel_len) of every head.
 struct MergeArgs {
-  const float* o_parts;   // [n_parts, heads * S, D]
-  const float* lse_parts; // [n_parts, heads * S]
+  const float* o_parts;   // [slots, heads * S, D]
+  const float* lse_parts; // [slots, heads * S]
   void* out;              // [heads * S, D] storage dtype
   float* lse;             // [heads * S]
   int64_t rows;           // heads * sel_len rows are merged
-  int64_t part_stride_rows;  // rows between consecutive parts (>= heads * S)
-  int n_parts;
-  int first_wrapped;      // active parts: part 0 and parts first_wrapped .. n_parts-1 (1 = all);
-                          // inactive parts are never read
+  int64_t part_stride_rows;  // rows between consecutive slots (>= heads * S)
+  uint64_t active;        // bit s set: slot s holds a partial for these rows; other slots are never read
   int S;                  // rows per head
   int sel_start, sel_len; // row range within a head
 };

@@ -137,35 +137,35 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 31, h = lane >> 5;
 
-  // workgroup -> (head, rank, q tile), XCD-aware as in block_attention_kernel
+  // workgroup -> (head, work item, q tile).  blockIdx mod 8 is the XCD: the q tiles of a
+  // (head, item) group stay on one XCD and share its K and V in that L2.  Groups are
+  // head-major (the items of a head run together) over an ODD item count (the host pads by
+  // one empty item if needed): an XCD takes every 8th group and so cycles through all items;
+  // with a count sharing a factor with 8 it would get the same few items for every head,
+  // and items differ in cost.
   const int q_tiles = a.q_tiles_max;
-  const int groups = a.n_active * a.BH;
+  const int n_pad = a.n_items | 1;
+  const int groups = n_pad * a.BH;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int group = (slot / q_tiles) * 8 + xcd;
   if (group >= groups) return;
-  const int ridx = group % a.n_active, bh = group / a.n_active;
-  int r = a.rank_base + ridx, step = a.step;
-  if (a.pairs) {
-    const int pr = a.pairs[ridx];
-    r = pr >> 16;
-    step = pr & 0xffff;
-  }
-  int j = r + step;
-  if (j >= a.P) j -= a.P;
-  if (a.causal && j > r) return;
-  const bool diag = a.causal && (j == r);
-  const int q_start = a.rank_start[r], q_len = a.rank_start[r + 1] - q_start;
-  const int kv_start = a.rank_start[j], kv_len = a.rank_start[j + 1] - kv_start;
+  const int bh = group / n_pad, item = group % n_pad;
+  if (item >= a.n_items) return;
+  const WorkItem w = a.items[item];
+  const bool diag = w.diag_off >= 0;
+  const int q_start = w.q_start, q_len = w.q_len;
+  const int kv_start = w.kv_start, kv_len = w.kv_len;
   int qt = slot % q_tiles;
-  if (qt * BM >= q_len) return;  // ranks shorter than the longest one
-  if (diag) qt = q_len / BM - 1 - qt;
-  const int n_tiles = diag ? ((qt + 1) * BM) / BN : kv_len / BN;
-  const int first_masked = diag ? (qt * BM) / BN : n_tiles;  // tiles >= this need the causal mask
+  if (qt * BM >= q_len) return;  // items shorter than the longest one
+  if (diag) qt = q_len / BM - 1 - qt;  // most keys first
+  const int diag_rows = w.diag_off + qt * BM;  // keys below this local index are visible to the whole q tile
+  const int n_tiles = diag ? (diag_rows + BM) / BN : kv_len / BN;
+  const int first_masked = diag ? diag_rows / BN : n_tiles;  // tiles >= this need the causal mask
 
   const int64_t head_off = (int64_t)bh * a.bh_stride;
   // grouped-query attention: query head h of a batch entry reads KV head h / kv_group
   const int kv_bh = (bh / a.heads) * (a.heads / a.kv_group) + (bh % a.heads) / a.kv_group;
-  const int64_t kv_head_off = (int64_t)kv_bh * a.bh_stride;
+  const int64_t kv_head_off = (int64_t)kv_bh * a.kv_bh_stride;
   const char* qbase = (const char*)a.q + (head_off + (int64_t)(q_start + qt * BM) * D) * 2;
   const char* kbase = (const char*)a.k + (kv_head_off + (int64_t)kv_start * D) * 2;
   const char* vbase = (const char*)a.v + (kv_head_off + (int64_t)kv_start * D) * 2;
@@ -246,10 +246,10 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
     }
   };
   auto mask_tile = [&](f32x16(&sacc)[QB], int t) {
-    if (t >= first_masked) {  // diagonal chunk pair: key visible iff key_local <= query_local
+    if (t >= first_masked) {  // key visible iff key_local <= query_local + diag_off
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
-        const int lim = qt * BM + 32 * QB * wave + 32 * qb + n - t * BN - 4 * h;
+        const int lim = diag_rows + 32 * QB * wave + 32 * qb + n - t * BN - 4 * h;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int key = 8 * (e >> 2) + (e & 3);
@@ -427,7 +427,7 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
     const float l = cross_half_sum((ls[qb][0] + ls[qb][1]) + (ls[qb][2] + ls[qb][3]));
     const float inv = (l > 0.f) ? 1.f / l : 0.f;
     const int row_g = q_start + qt * BM + 32 * QB * wave + 32 * qb + n;
-    const int64_t slot_rows = a.pairs ? (int64_t)step * a.part_stride_rows : 0;
+    const int64_t slot_rows = (int64_t)(w.slot - a.slot_bias) * a.part_stride_rows;
     float* orow = a.o_part + (slot_rows + (int64_t)bh * a.S + row_g) * D;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
@@ -472,29 +472,27 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
   if (row >= a.rows) return;
   row = (row / a.sel_len) * a.S + a.sel_start + row % a.sel_len;
   const int c8 = threadIdx.x % TPR;
-  // active parts of this row: part 0 and parts first_wrapped .. n_parts-1 (ring), or all
-  const int first_wrapped = a.first_wrapped;
-  const int n_act = a.n_parts - first_wrapped + 1;
-  auto part_of = [&](int i) { return i == 0 ? 0 : first_wrapped + i - 1; };
+  // active slots of these rows: the set bits of a.active, visited in ascending order
   const float* lse_row = a.lse_parts + row;
   const float* o_row = a.o_parts + row * D + c8 * 8;
   const int64_t lse_stride = a.part_stride_rows, o_stride = a.part_stride_rows * D;
 
   float mx = -INFINITY;
-  for (int i = 0; i < n_act; ++i) mx = fmaxf(mx, lse_row[part_of(i) * lse_stride]);
+  for (uint64_t rest = a.active; rest; rest &= rest - 1) mx = fmaxf(mx, lse_row[__builtin_ctzll(rest) * lse_stride]);
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   float wsum = 0.f;
   if (mx != -INFINITY) {
-    // four parts per iteration: all their loads are issued before the first is consumed
-    int i = 0;
-    for (; i + 4 <= n_act; i += 4) {
+    // four slots per iteration: all their loads are issued before the first is consumed
+    uint64_t rest = a.active;
+    while (__builtin_popcountll(rest) >= 4) {
       float L[4];
       f32x4 x0[4], x1[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int64_t s = part_of(i + u);
+        const int64_t s = __builtin_ctzll(rest);
+        rest &= rest - 1;
         L[u] = lse_row[s * lse_stride];
         x0[u] = *(const f32x4*)(o_row + s * o_stride);
         x1[u] = *(const f32x4*)(o_row + s * o_stride + 4);
@@ -511,8 +509,8 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
         }
       }
     }
-    for (; i < n_act; ++i) {
-      const int64_t s = part_of(i);
+    for (; rest; rest &= rest - 1) {
+      const int64_t s = __builtin_ctzll(rest);
       const float Ls = lse_row[s * lse_stride];
       const float w = __expf(Ls - mx);
       const f32x4 x0 = *(const f32x4*)(o_row + s * o_stride), x1 = *(const f32x4*)(o_row + s * o_stride + 4);
@@ -534,10 +532,12 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
 
 // ---- host launchers -----------------------------------------------------------------
 hipError_t launch_block_step(const BlockStepArgs& a, int dtype, int dim, hipStream_t stream) {
-  if (a.n_active <= 0) return hipSuccess;
+  if (a.n_items <= 0) return hipSuccess;
   const int q_tiles = a.q_tiles_max;
-  const int groups = a.n_active * a.BH;
-  const unsigned grid = (unsigned)(((groups + 7) / 8) * 8 * q_tiles);
+  const int64_t groups = (int64_t)(a.n_items | 1) * a.BH;  // odd item count, see the kernel
+  const int64_t blocks = ((groups + 7) / 8) * 8 * q_tiles;
+  if (q_tiles <= 0 || blocks > INT32_MAX) return hipErrorInvalidValue;
+  const unsigned grid = (unsigned)blocks;
   if (dtype == 0 && dim == 64) block_attention_kernel<0, 64><<<grid, 256, 0, stream>>>(a);
   else if (dtype == 0 && dim == 128) block_attention_kernel<0, 128><<<grid, 256, 0, stream>>>(a);
   else if (dtype == 1 && dim == 64) block_attention_kernel<1, 64><<<grid, 256, 0, stream>>>(a);

@@ -14,9 +14,9 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 OK, E_NULL, E_NPES, E_DIM, E_DTYPE, E_SEQLEN, E_SHAPE, E_WS, E_RANK, E_PLAN, E_HIP, E_ALLOC, E_ALIGN = range(13)
 
 
-def params(npes=2, seqlen=(128, 128), dim=64, batch=1, heads=1, dtype=0, causal=0, flags=0, scale=0.0, kv_heads=0):
+def params(npes=2, seqlen=(128, 128), dim=64, batch=1, heads=1, dtype=0, causal=0, flags=0, scale=0.0, kv_heads=0, layout=0):
     arr = (ctypes.c_int * max(1, len(seqlen)))(*seqlen)
-    p = RingattnParams(npes, ctypes.cast(arr, _lib.c_int_p), dim, scale, batch, heads, dtype, causal, flags, kv_heads)
+    p = RingattnParams(npes, ctypes.cast(arr, _lib.c_int_p), dim, scale, batch, heads, dtype, causal, flags, kv_heads, layout)
     p._keep = arr
     return p
 
@@ -73,6 +73,8 @@ def test_parameter_validation(ralib):
     assert create(params(scale=float("nan"))) == E_SHAPE
     assert create(params(heads=8, kv_heads=3)) == E_SHAPE     # kv_heads must divide heads
     assert create(params(heads=8, kv_heads=-2)) == E_SHAPE
+    assert create(params(layout=2)) == E_SHAPE                # unknown layout
+    assert create(params(layout=1, causal=1)) == E_SEQLEN     # zigzag halves must be multiples of 128
     for bad in (params(npes=0), params(dim=7), params(seqlen=(64, 64))):
         assert wb(ctypes.byref(bad)) == 0
     assert wb(None) == 0
@@ -131,3 +133,84 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libringattn.so"))
     with pytest.raises(RuntimeError, match="has not been built"):
         _lib.load()
+
+
+def _plan_on_host(ralib, p):
+    # the workspace of a plan is never touched on the host: any aligned address will do
+    need = ralib.ringattn_workspace_bytes(ctypes.byref(p))
+    h = ctypes.c_void_p()
+    assert ralib.ringattn_plan_create(ctypes.byref(p), ctypes.c_void_p(1 << 20), need, ctypes.byref(h)) == OK
+    return h
+
+
+def _work_items(ralib, h, step):
+    n = ctypes.c_int()
+    assert ralib.ringattn_plan_work_items(h, step, None, 0, ctypes.byref(n)) == OK
+    items = (_lib.RingattnWorkItem * max(1, n.value))()
+    assert ralib.ringattn_plan_work_items(h, step, items, n.value, ctypes.byref(n)) == OK
+    return [items[i] for i in range(n.value)]
+
+
+@pytest.mark.parametrize("seqlen,causal,layout", [
+    ((256, 256, 256, 256), 0, 0), ((256, 256, 256, 256), 1, 0), ((256, 256, 256, 256), 1, 1), ((256, 256, 256, 256), 0, 1),
+    ((256, 768, 512), 1, 1), ((512, 256, 256, 768, 256), 1, 1), ((128, 384, 256), 1, 0), ((512,), 1, 1),
+    ((256,) * 9, 1, 1), ((256,) * 16, 1, 0), ((256,) * 16, 1, 1),
+])
+def test_schedule_covers_every_visible_pair_exactly_once(ralib, seqlen, causal, layout):
+    from ringattention_amd.api import zigzag_order
+    P, S = len(seqlen), sum(seqlen)
+    h = _plan_on_host(ralib, params(npes=P, seqlen=seqlen, causal=causal, layout=layout))
+    start = np.concatenate([[0], np.cumsum(seqlen)])
+    rank_of = np.repeat(np.arange(P), seqlen)
+    pos = zigzag_order(seqlen) if layout == 1 else np.arange(S)    # sequence position of memory row i
+    want = (pos[None, :] <= pos[:, None]) if causal else np.ones((S, S), bool)
+
+    def coverage(items):
+        cover = np.zeros((S, S), np.int32)
+        slots = [set() for _ in range(S)]
+        for w in items:
+            assert w.q_len > 0 and w.kv_len > 0 and all(x % 128 == 0 for x in (w.q_start, w.q_len, w.kv_start, w.kv_len))
+            r = rank_of[w.q_start]
+            j = (r + w.slot) % P                                    # ring discipline: step s visits rank (r + s) mod P
+            assert start[r] <= w.q_start and w.q_start + w.q_len <= start[r + 1]
+            assert start[j] <= w.kv_start and w.kv_start + w.kv_len <= start[j + 1]
+            vis = np.ones((w.q_len, w.kv_len), bool)
+            if w.diag_off >= 0:
+                assert w.diag_off + w.q_len <= w.kv_len
+                vis = np.arange(w.kv_len)[None, :] <= np.arange(w.q_len)[:, None] + w.diag_off
+            cover[w.q_start:w.q_start + w.q_len, w.kv_start:w.kv_start + w.kv_len] += vis
+            for row in range(w.q_start, w.q_start + w.q_len, 128):
+                assert w.slot not in slots[row]                     # one partial per row and slot
+                slots[row].add(w.slot)
+        return cover, slots
+
+    cover, slots = coverage(_work_items(ralib, h, -1))
+    assert np.array_equal(cover, want.astype(np.int32))
+    per_step = [w for s in range(P) for w in _work_items(ralib, h, s)]
+    assert all(w.slot == s for s in range(P) for w in _work_items(ralib, h, s))
+    cover2, _ = coverage(per_step)
+    assert np.array_equal(cover2, cover)
+    # merge regions: a partition of the rows, each with exactly the slots that were written
+    n = ctypes.c_int()
+    cap = 4 * P
+    st, ln, act = (ctypes.c_int * cap)(), (ctypes.c_int * cap)(), (ctypes.c_uint64 * cap)()
+    assert ralib.ringattn_plan_merge_regions(h, st, ln, act, cap, ctypes.byref(n)) == OK
+    seen = np.zeros(S, np.int32)
+    for i in range(n.value):
+        seen[st[i]:st[i] + ln[i]] += 1
+        for row in range(st[i], st[i] + ln[i], 128):
+            assert {s for s in range(64) if act[i] >> s & 1} == slots[row]
+    assert np.all(seen == 1)
+    if causal and layout == 1 and len(set(seqlen)) == 1:           # zigzag: every rank does the same work
+        work = [want[start[r]:start[r + 1]].sum() for r in range(P)]
+        assert max(work) - min(work) <= seqlen[0]                   # equal up to the diagonal's own width
+    assert ralib.ringattn_plan_destroy(h) == OK
+
+
+def test_zigzag_order_small_case():
+    from ringattention_amd.api import zigzag_order
+    # two ranks of 4 rows: rank 0 holds positions 0,1 and 6,7; rank 1 holds 2,3 and 4,5
+    assert zigzag_order([4, 4]).tolist() == [0, 1, 6, 7, 2, 3, 4, 5]
+    o = zigzag_order([256, 768, 512])
+    assert sorted(o.tolist()) == list(range(1536))
+    assert o[:128].tolist() == list(range(128)) and o[128] == 1536 - 128   # rank 0: first low half, last high half

@@ -166,6 +166,81 @@ def test_grouped_query_heads(oracle, causal):
     check_rows(oracle, w, q, k_rep, v_rep, out, lse, np.arange(w.rows))
 
 
+@pytest.mark.parametrize("seqlen,B,H,d,dtype,hkv", [
+    ((512, 512, 512, 512), 1, 2, 128, "bf16", 0),
+    ((256, 768, 512), 2, 3, 64, "fp16", 0),           # unequal ranks, odd rank count
+    ((1024,), 1, 2, 128, "fp16", 0),                  # one rank: zigzag degenerates to the plain causal mask
+    ((256,) * 8, 1, 4, 128, "bf16", 2),               # with grouped-query heads
+])
+def test_zigzag_layout(oracle, seqlen, B, H, d, dtype, hkv):
+    # The sequence is generated in sequence order, stored in zigzag memory order, and the
+    # result (brought back to sequence order) must equal causal attention over the sequence.
+    P, S = len(seqlen), sum(seqlen)
+    w = Workload("zigzag", B, H, d, 1, S, dtype, 91, True)
+    q, k, v = api.make_qkv_bits(w)
+    if hkv:
+        _, k, v = api.make_qkv_bits(Workload("zigzag_kv", B, hkv, d, 1, S, dtype, 92, True))
+    order = api.zigzag_order(seqlen)
+    inv = torch.from_numpy(np.argsort(order)).cuda()
+    qd, kd, vd = (to_dev(np.ascontiguousarray(x[:, :, order]), dtype) for x in (q, k, v))
+    plan = api.RingAttention(P, list(seqlen), d, B, H, dtype, True, kv_heads=hkv, layout="zigzag")
+    out, lse = plan.forward(qd, kd, vd)
+    torch.cuda.synchronize()
+    out_seq, lse_seq = out[:, :, inv].contiguous(), lse[:, :, inv].contiguous()
+    k_full, v_full = ((np.repeat(x, H // hkv, axis=1) if hkv else x) for x in (k, v))
+    check_rows(oracle, w, q, k_full, v_full, out_seq, lse_seq, np.arange(w.rows))
+    # step by step through the C ABI: the same items, so the same bits
+    o_parts = torch.zeros((P, B, H, S, d), dtype=torch.float32, device="cuda")
+    lse_parts = torch.full((P, B, H, S), float("-inf"), dtype=torch.float32, device="cuda")
+    for s in range(P):
+        plan.block_forward(s, qd, kd, vd, o_parts[s], lse_parts[s])
+    out2, lse2 = plan.merge_ring(o_parts, lse_parts)
+    torch.cuda.synchronize()
+    assert torch.equal(out2, out) and torch.equal(lse2, lse)
+    # low halves never see a later rank: those (row, step) partials stay untouched
+    start = np.concatenate([[0], np.cumsum(seqlen)])
+    for r in range(P):
+        for s in range(1, P):
+            low = lse_parts[s, :, :, start[r]:start[r] + seqlen[r] // 2]
+            assert bool(torch.isinf(low).all()) == ((r + s) % P > r)
+    plan.close()
+
+
+def test_zigzag_without_mask_equals_contiguous():
+    w = Workload("zz_nomask", 1, 2, 128, 4, 256, "bf16", 93, False)
+    q, k, v = (to_dev(x, w.dtype) for x in api.make_qkv_bits(w))
+    res = []
+    for layout in ("contiguous", "zigzag"):
+        plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, False, layout=layout)
+        res.append(plan.forward(q, k, v))
+        torch.cuda.synchronize()
+        plan.close()
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
+
+
+def test_zigzag_cfg4_sampled_rows(oracle):
+    w = WORKLOADS["cfg4"]
+    q, k, v = api.make_qkv_bits(w)
+    seqlen = [w.chunk] * w.npes
+    order = api.zigzag_order(seqlen)
+    inv = np.argsort(order)
+    order_d = torch.from_numpy(order).cuda()
+    qd, kd, vd = (to_dev(x, w.dtype)[:, :, order_d].contiguous() for x in (q, k, v))
+    plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, True, layout="zigzag")
+    out, lse = plan.forward(qd, kd, vd)
+    torch.cuda.synchronize()
+    plan.close()
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    rows_seq = sample_rows(w, 384)                                  # (head, sequence position) pairs
+    head, posn = rows_seq // w.seq, rows_seq % w.seq
+    rows_mem = torch.from_numpy(head * w.seq + inv[posn]).cuda()
+    o_ref, l_ref = oracle.attention_rows(q, k, v, w.dtype, causal=True, rows=rows_seq)
+    o_gpu = out.reshape(-1, w.dim)[rows_mem].double().cpu().numpy()
+    l_gpu = lse.reshape(-1)[rows_mem].double().cpu().numpy()
+    assert np.abs(o_gpu - o_ref).max() <= O_TOL
+    assert (np.abs(l_gpu - l_ref) / np.maximum(np.abs(l_ref), 1e-3)).max() <= LSE_RTOL
+
+
 def test_explicit_softmax_scale(oracle):
     w = Workload("scale", 1, 2, 64, 2, 256, "fp16", 31, False)
     q, k, v = api.make_qkv_bits(w)
