@@ -30,7 +30,7 @@ extern "C" {
 #define RINGATTN_ERR_NPES 2        /* npes < 1 or above RINGATTN_MAX_NPES */
 #define RINGATTN_ERR_DIM 3         /* dim not in {64, 128} */
 #define RINGATTN_ERR_DTYPE 4       /* dtype not fp16 / bf16 */
-#define RINGATTN_ERR_SEQLEN 5      /* a per-rank length is not a positive multiple of 128 (256 with the zigzag layout), or max_seq is below it */
+#define RINGATTN_ERR_SEQLEN 5      /* a per-rank length is not positive (or odd, with the zigzag layout), or max_seq is below it */
 #define RINGATTN_ERR_SHAPE 6       /* batch or heads < 1, kv_heads does not divide heads, unknown layout, sizes overflow */
 #define RINGATTN_ERR_WORKSPACE 7   /* caller workspace missing or too small */
 #define RINGATTN_ERR_RANK 8        /* mype / step outside [0, npes) */
@@ -43,7 +43,9 @@ extern "C" {
 #define RINGATTN_DTYPE_BF16 1
 
 #define RINGATTN_MAX_NPES 64
-#define RINGATTN_TILE 128          /* per-rank lengths must be multiples of this; they may differ between ranks */
+#define RINGATTN_TILE 128          /* query rows per workgroup: per-rank lengths may be any positive number and may differ between
+                                      ranks (the tail predication the reference leaves open, csrc/ring_attention.cu:143-145);
+                                      multiples of this waste no part of a tile */
 
 #define RINGATTN_FLAG_GRAPH 1      /* capture the step loop + merge in a hipGraph and replay it */
 
@@ -54,7 +56,7 @@ extern "C" {
  * halves of ranks 0..npes-1 come first and then the high halves of ranks npes-1..0, so that
  * under the causal mask every rank has the same amount of work (with CONTIGUOUS rank r has
  * r + 1 visible chunks).  The reference has no causal mask and therefore no such layout; it
- * only matters when `causal` is set.  Per-rank lengths must then be multiples of 256.
+ * only matters when `causal` is set.  Per-rank lengths must then be even.
  */
 #define RINGATTN_LAYOUT_CONTIGUOUS 0
 #define RINGATTN_LAYOUT_ZIGZAG 1

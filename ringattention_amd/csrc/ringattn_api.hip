@@ -58,12 +58,14 @@ int validate(const ringattn_params* p, Derived* d) {
   if (p->batch < 1 || p->heads < 1) return RINGATTN_ERR_SHAPE;
   if (p->kv_heads < 0 || (p->kv_heads > 0 && p->heads % p->kv_heads != 0)) return RINGATTN_ERR_SHAPE;
   if (p->layout != RINGATTN_LAYOUT_CONTIGUOUS && p->layout != RINGATTN_LAYOUT_ZIGZAG) return RINGATTN_ERR_SHAPE;
-  const int tile = p->layout == RINGATTN_LAYOUT_ZIGZAG ? 2 * RINGATTN_TILE : RINGATTN_TILE;
+  // any positive length (the zigzag layout halves it, so even there); multiples of
+  // RINGATTN_TILE waste no part of a tile
+  const int granule = p->layout == RINGATTN_LAYOUT_ZIGZAG ? 2 : 1;
   int64_t S = 0;
   int max_len = 0;
   for (int r = 0; r < p->npes; ++r) {
     const int c = p->h_seqlen[r];
-    if (c <= 0 || c % tile != 0) return RINGATTN_ERR_SEQLEN;
+    if (c <= 0 || c % granule != 0) return RINGATTN_ERR_SEQLEN;
     S += c;
     if (c > max_len) max_len = c;
   }
@@ -270,7 +272,7 @@ void build_schedule(ringattn_plan* pl) {
   pl->step_begin.push_back((int)pl->h_items.size());
   int longest = 0;
   for (const auto& w : pl->h_items) longest = w.q_len > longest ? w.q_len : longest;
-  pl->q_tiles_max = longest / ringattn::kBlockM;
+  pl->q_tiles_max = (longest + ringattn::kBlockM - 1) / ringattn::kBlockM;
 }
 
 int ensure_streams(ringattn_plan* pl) {
@@ -587,11 +589,12 @@ int ringattn_ring_attention(const void* q, const void* k, const void* v, void* o
   // per-call scratch, like the reference's per-call allocations (:383-394) but freed
   float* ws = nullptr;
   const size_t table_bytes = (size_t)n_parts * sizeof(ringattn::WorkItem);
-  RA_HIP(hipMalloc((void**)&ws, (size_t)n_parts * c * (size_t)(dim + 1) * sizeof(float) + (size_t)c * sizeof(float) + table_bytes));
+  const size_t lse_floats = ((size_t)(n_parts + 1) * c + 7) & ~(size_t)7;  // keeps the item table 32-byte aligned
+  RA_HIP(hipMalloc((void**)&ws, ((size_t)n_parts * c * dim + lse_floats) * sizeof(float) + table_bytes));
   float* o_parts = ws;
   float* lse_parts = ws + (size_t)n_parts * c * dim;
   float* lse_tmp = lse_parts + (size_t)n_parts * c;
-  ringattn::WorkItem* d_items = (ringattn::WorkItem*)(lse_tmp + c);  // 16-byte aligned: c is a multiple of 128
+  ringattn::WorkItem* d_items = (ringattn::WorkItem*)(lse_parts + lse_floats);
   hipError_t e = hipMemcpy(d_items, items.data(), table_bytes, hipMemcpyHostToDevice);
   if (e != hipSuccess) rc = hip_fail(e);
   if (rc == RINGATTN_OK) {
@@ -604,7 +607,7 @@ int ringattn_ring_attention(const void* q, const void* k, const void* v, void* o
     a.lse_part = lse_parts;
     a.items = d_items;
     a.n_items = n_parts;
-    a.q_tiles_max = c / ringattn::kBlockM;
+    a.q_tiles_max = (c + ringattn::kBlockM - 1) / ringattn::kBlockM;
     a.bh_stride = (int64_t)c * dim;
     a.part_stride_rows = c;
     a.S = c;
@@ -625,7 +628,7 @@ const char* ringattn_strerror(int code) {
     case RINGATTN_ERR_NPES: return "npes out of range";
     case RINGATTN_ERR_DIM: return "dim must be 64 or 128";
     case RINGATTN_ERR_DTYPE: return "dtype must be fp16 (0) or bf16 (1)";
-    case RINGATTN_ERR_SEQLEN: return "per-rank sequence lengths must be positive multiples of 128 (256 with the zigzag layout), and max_seq at least the longest";
+    case RINGATTN_ERR_SEQLEN: return "per-rank sequence lengths must be positive (even with the zigzag layout), and max_seq at least the longest";
     case RINGATTN_ERR_SHAPE: return "batch/heads/kv_heads/layout/scale invalid or sizes overflow";
     case RINGATTN_ERR_WORKSPACE: return "workspace too small";
     case RINGATTN_ERR_RANK: return "rank or step outside [0, npes)";

@@ -157,10 +157,17 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   const int kv_start = w.kv_start, kv_len = w.kv_len;
   int qt = slot % q_tiles;
   if (qt * BM >= q_len) return;  // items shorter than the longest one
-  if (diag) qt = q_len / BM - 1 - qt;  // most keys first
+  if (diag) qt = (q_len + BM - 1) / BM - 1 - qt;  // most keys first
   const int diag_rows = w.diag_off + qt * BM;  // keys below this local index are visible to the whole q tile
-  const int n_tiles = diag ? (diag_rows + BM) / BN : kv_len / BN;
-  const int first_masked = diag ? diag_rows / BN : n_tiles;  // tiles >= this need the causal mask
+  // Lengths need not be multiples of the tile sizes (the predication the reference leaves as
+  // a TODO, csrc/ring_attention.cu:143-145).  The last key tile may reach beyond the KV range:
+  // its loads are clamped to the last valid row and its surplus keys masked.  Query rows
+  // beyond the range are computed on a copy of the last valid row and not stored.
+  const int kv_tiles = (kv_len + BN - 1) / BN;
+  const int kv_tail = (kv_len % BN) ? kv_len / BN : -1;  // the tile with surplus keys, if any
+  const int n_tiles = diag ? min(kv_tiles, (diag_rows + BM + BN - 1) / BN) : kv_tiles;
+  // tiles >= first_masked need a mask (causal diagonal or surplus keys)
+  const int first_masked = min(diag ? diag_rows / BN : n_tiles, kv_tail >= 0 ? kv_tail : n_tiles);
 
   const int64_t head_off = (int64_t)bh * a.bh_stride;
   // grouped-query attention: query head h of a batch entry reads KV head h / kv_group
@@ -174,7 +181,8 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   s16x8 qf[QB][KS];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    const char* qrow = qbase + (int64_t)(32 * QB * wave + 32 * qb + n) * ROWB + h * 16;
+    const int ql = min(qt * BM + 32 * QB * wave + 32 * qb + n, q_len - 1) - qt * BM;
+    const char* qrow = qbase + (int64_t)ql * ROWB + h * 16;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qf[qb][ks] = *(const s16x8*)(qrow + ks * 32);
   }
@@ -218,18 +226,36 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   f32x16 s_even[QB], s_odd[QB];
   s16x8 pf[QB][2];
 
-  auto issue_k = [&](int t) {
+  // bytes to step back so that a row of tile kv_tail beyond the KV range reads the last valid row
+  auto surplus = [&](int i) {
+    const int row = ((wave * LD + i) * 64 + lane) / CPR;
+    return max(0, kv_tail * BN + row - (kv_len - 1)) * ROWB;
+  };
+  // `checked`: the tile may be kv_tail (steady blocks never issue that one)
+  auto issue_k = [&](int t, auto checked) {
     const char* kt = kbase + (int64_t)t * TILE;
     const unsigned kd = __builtin_amdgcn_readfirstlane(smem_base + (t & (NBUF - 1)) * TILE + wave * (LD * 1024));
+    if (decltype(checked)::value && t == kv_tail) {
 #pragma unroll
-    for (int i = 0; i < LD; ++i) load_lds_16(kt, goff_k[i], kd + i * 1024);
+      for (int i = 0; i < LD; ++i) load_lds_16(kt, goff_k[i] - surplus(i), kd + i * 1024);
+    } else {
+#pragma unroll
+      for (int i = 0; i < LD; ++i) load_lds_16(kt, goff_k[i], kd + i * 1024);
+    }
   };
-  auto issue_v = [&](int t) {
+  auto issue_v = [&](int t, auto checked) {
     const char* vt = vbase + (int64_t)t * TILE;
     const unsigned vd = __builtin_amdgcn_readfirstlane(smem_base + (NBUF + (t & (NBUF - 1))) * TILE + wave * (LD * 1024));
+    if (decltype(checked)::value && t == kv_tail) {
 #pragma unroll
-    for (int i = 0; i < LD; ++i) load_lds_16(vt, goff_v[i], vd + i * 1024);
+      for (int i = 0; i < LD; ++i) load_lds_16(vt, goff_v[i] - surplus(i), vd + i * 1024);
+    } else {
+#pragma unroll
+      for (int i = 0; i < LD; ++i) load_lds_16(vt, goff_v[i], vd + i * 1024);
+    }
   };
+  constexpr std::true_type kChecked{};
+  constexpr std::false_type kUnchecked{};
   // S^T = K Q^T of one 32-key tile (csrc/ring_attention.cu:565); each K fragment feeds all
   // QB query blocks of the wave
   auto qk = [&](f32x16(&sacc)[QB], int kslot) {
@@ -246,10 +272,11 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
     }
   };
   auto mask_tile = [&](f32x16(&sacc)[QB], int t) {
-    if (t >= first_masked) {  // key visible iff key_local <= query_local + diag_off
+    if (t >= first_masked) {  // key visible iff inside the KV range and key_local <= query_local + diag_off
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
-        const int lim = diag_rows + 32 * QB * wave + 32 * qb + n - t * BN - 4 * h;
+        int lim = kv_len - 1 - t * BN - 4 * h;
+        if (diag) lim = min(lim, diag_rows + 32 * QB * wave + 32 * qb + n - t * BN - 4 * h);
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int key = 8 * (e >> 2) + (e & 3);
@@ -346,14 +373,14 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
       if ((SLOT & 1) == 0) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        issue_k(u + 3);
+        issue_k(u + 3, kUnchecked);
       } else {
-        issue_v(u + 1);
+        issue_v(u + 1, kUnchecked);
       }
       qk(nxt, (SLOT + 1) & 3);
       exponentials(cur);
-      if ((SLOT & 1) == 0) issue_k(u + 4);
-      else issue_v(u + 2);
+      if ((SLOT & 1) == 0) issue_k(u + 4, kUnchecked);
+      else issue_v(u + 2, kUnchecked);
       pv_product(SLOT);
       tile_maxes(nxt, cand);
       // scheduling hint: in the first half of the block every MFMA is preceded by one and
@@ -369,10 +396,10 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
       if ((u & 1) == 0) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (u + 3 < n_tiles) issue_k(u + 3);
-        if (u + 4 < n_tiles) issue_k(u + 4);
-        if (u + 2 < n_tiles) issue_v(u + 2);
-        if (u + 3 < n_tiles) issue_v(u + 3);
+        if (u + 3 < n_tiles) issue_k(u + 3, kChecked);
+        if (u + 4 < n_tiles) issue_k(u + 4, kChecked);
+        if (u + 2 < n_tiles) issue_v(u + 2, kChecked);
+        if (u + 3 < n_tiles) issue_v(u + 3, kChecked);
       }
       if (u + 1 < n_tiles) {
         qk(nxt, (u + 1) & 3);
@@ -388,13 +415,13 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   };
 
   __builtin_amdgcn_s_waitcnt(0);  // retire the Q loads with a wait the compiler can see
-  issue_k(0);
+  issue_k(0, kChecked);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  if (n_tiles > 1) issue_k(1);
-  if (n_tiles > 2) issue_k(2);
-  issue_v(0);
-  if (n_tiles > 1) issue_v(1);
+  if (n_tiles > 1) issue_k(1, kChecked);
+  if (n_tiles > 2) issue_k(2, kChecked);
+  issue_v(0, kChecked);
+  if (n_tiles > 1) issue_v(1, kChecked);
   {
     float cand[QB];
     qk(s_even, 0);
@@ -407,8 +434,9 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   using C1 = std::integral_constant<int, 1>;
   using C2 = std::integral_constant<int, 2>;
   using C3 = std::integral_constant<int, 3>;
-  // a steady pair (u, u+1), u even, needs u + 4 < n_tiles and u + 2 < first_masked
-  const int n_steady = min(n_tiles - 4, first_masked - 2);  // pairs starting at u < n_steady
+  // a steady pair (u, u+1), u even, needs u + 4 < n_tiles (and that tile not to be kv_tail)
+  // and u + 2 < first_masked
+  const int n_steady = min(n_tiles - 4 - (kv_tail >= 0 ? 1 : 0), first_masked - 2);  // pairs starting at u < n_steady
   int u = 0;
   for (; u + 2 < n_steady; u += 4) {
     block(C0{}, std::true_type{}, u);
@@ -426,7 +454,9 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   for (int qb = 0; qb < QB; ++qb) {
     const float l = cross_half_sum((ls[qb][0] + ls[qb][1]) + (ls[qb][2] + ls[qb][3]));
     const float inv = (l > 0.f) ? 1.f / l : 0.f;
-    const int row_g = q_start + qt * BM + 32 * QB * wave + 32 * qb + n;
+    const int row_l = qt * BM + 32 * QB * wave + 32 * qb + n;
+    if (row_l >= q_len) continue;  // a row beyond the query range
+    const int row_g = q_start + row_l;
     const int64_t slot_rows = (int64_t)(w.slot - a.slot_bias) * a.part_stride_rows;
     float* orow = a.o_part + (slot_rows + (int64_t)bh * a.S + row_g) * D;
 #pragma unroll

@@ -64,8 +64,9 @@ def test_parameter_validation(ralib):
         assert create(params(dim=bad_dim)) == E_DIM
     assert create(params(dtype=2)) == E_DTYPE
     assert create(params(dtype=-1)) == E_DTYPE
-    assert create(params(seqlen=(128, 200))) == E_SEQLEN      # one rank not a multiple of the tile
-    assert create(params(seqlen=(100, 100))) == E_SEQLEN
+    assert wb(ctypes.byref(params(seqlen=(128, 200)))) == 2 * 328 * 65 * 4   # nor need they be multiples of the tile
+    assert wb(ctypes.byref(params(seqlen=(1, 3)))) == 2 * 4 * 65 * 4
+    assert create(params(seqlen=(0, 128))) == E_SEQLEN
     assert create(params(seqlen=(0, 0))) == E_SEQLEN
     assert create(params(seqlen=(-128, -128))) == E_SEQLEN
     assert create(params(batch=0)) == E_SHAPE
@@ -74,8 +75,8 @@ def test_parameter_validation(ralib):
     assert create(params(heads=8, kv_heads=3)) == E_SHAPE     # kv_heads must divide heads
     assert create(params(heads=8, kv_heads=-2)) == E_SHAPE
     assert create(params(layout=2)) == E_SHAPE                # unknown layout
-    assert create(params(layout=1, causal=1)) == E_SEQLEN     # zigzag halves must be multiples of 128
-    for bad in (params(npes=0), params(dim=7), params(seqlen=(64, 64))):
+    assert create(params(layout=1, causal=1, seqlen=(128, 129))) == E_SEQLEN     # zigzag halves a rank: even lengths
+    for bad in (params(npes=0), params(dim=7), params(seqlen=(64, -64))):
         assert wb(ctypes.byref(bad)) == 0
     assert wb(None) == 0
 
@@ -155,6 +156,7 @@ def _work_items(ralib, h, step):
     ((256, 256, 256, 256), 0, 0), ((256, 256, 256, 256), 1, 0), ((256, 256, 256, 256), 1, 1), ((256, 256, 256, 256), 0, 1),
     ((256, 768, 512), 1, 1), ((512, 256, 256, 768, 256), 1, 1), ((128, 384, 256), 1, 0), ((512,), 1, 1),
     ((256,) * 9, 1, 1), ((256,) * 16, 1, 0), ((256,) * 16, 1, 1),
+    ((100, 333, 1, 77), 1, 0), ((100, 333, 1, 77), 0, 0), ((130, 70, 2, 258), 1, 1), ((7,), 1, 0),   # ragged lengths
 ])
 def test_schedule_covers_every_visible_pair_exactly_once(ralib, seqlen, causal, layout):
     from ringattention_amd.api import zigzag_order
@@ -169,7 +171,7 @@ def test_schedule_covers_every_visible_pair_exactly_once(ralib, seqlen, causal, 
         cover = np.zeros((S, S), np.int32)
         slots = [set() for _ in range(S)]
         for w in items:
-            assert w.q_len > 0 and w.kv_len > 0 and all(x % 128 == 0 for x in (w.q_start, w.q_len, w.kv_start, w.kv_len))
+            assert w.q_len > 0 and w.kv_len > 0
             r = rank_of[w.q_start]
             j = (r + w.slot) % P                                    # ring discipline: step s visits rank (r + s) mod P
             assert start[r] <= w.q_start and w.q_start + w.q_len <= start[r + 1]
@@ -179,7 +181,7 @@ def test_schedule_covers_every_visible_pair_exactly_once(ralib, seqlen, causal, 
                 assert w.diag_off + w.q_len <= w.kv_len
                 vis = np.arange(w.kv_len)[None, :] <= np.arange(w.q_len)[:, None] + w.diag_off
             cover[w.q_start:w.q_start + w.q_len, w.kv_start:w.kv_start + w.kv_len] += vis
-            for row in range(w.q_start, w.q_start + w.q_len, 128):
+            for row in range(w.q_start, w.q_start + w.q_len):
                 assert w.slot not in slots[row]                     # one partial per row and slot
                 slots[row].add(w.slot)
         return cover, slots
@@ -198,7 +200,7 @@ def test_schedule_covers_every_visible_pair_exactly_once(ralib, seqlen, causal, 
     seen = np.zeros(S, np.int32)
     for i in range(n.value):
         seen[st[i]:st[i] + ln[i]] += 1
-        for row in range(st[i], st[i] + ln[i], 128):
+        for row in range(st[i], st[i] + ln[i]):
             assert {s for s in range(64) if act[i] >> s & 1} == slots[row]
     assert np.all(seen == 1)
     if causal and layout == 1 and len(set(seqlen)) == 1:           # zigzag: every rank does the same work

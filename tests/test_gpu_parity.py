@@ -150,6 +150,58 @@ def test_unequal_rank_lengths(oracle, seqlen, causal, d, dtype):
     plan.close()
 
 
+@pytest.mark.parametrize("seqlen,causal,d,dtype,layout", [
+    ((100, 333, 1, 77), False, 64, "fp16", "contiguous"),
+    ((100, 333, 1, 77), True, 128, "bf16", "contiguous"),
+    ((513,), True, 128, "fp16", "contiguous"),           # one rank, one row into a fifth q tile
+    ((31, 33), True, 64, "bf16", "contiguous"),          # shorter than one key tile / one more than it
+    ((1000, 24), False, 128, "bf16", "contiguous"),
+    ((130, 70, 2, 258), True, 128, "bf16", "zigzag"),
+    ((1, 1, 1), True, 64, "fp16", "contiguous"),
+])
+def test_ragged_lengths(oracle, seqlen, causal, d, dtype, layout):
+    # lengths that are no multiples of the 128-row q tile or the 32-key tile: the tail
+    # predication the reference leaves open (csrc/ring_attention.cu:143-145)
+    P, S, B, H = len(seqlen), sum(seqlen), 2, 2
+    w = Workload("ragged", B, H, d, 1, S, dtype, 95, causal)
+    q, k, v = api.make_qkv_bits(w)
+    order = api.zigzag_order(seqlen) if layout == "zigzag" else np.arange(S)
+    inv = torch.from_numpy(np.argsort(order)).cuda()
+    qd, kd, vd = (to_dev(np.ascontiguousarray(x[:, :, order]), dtype) for x in (q, k, v))
+    # output buffers with sentinel rows behind them: nothing may be written past the end
+    out_buf = torch.full((B * H * S + 64, d), 7.0, dtype=qd.dtype, device="cuda")
+    lse_buf = torch.full((B * H * S + 64,), 7.0, dtype=torch.float32, device="cuda")
+    out, lse = out_buf[:B * H * S].view(B, H, S, d), lse_buf[:B * H * S].view(B, H, S)
+    plan = api.RingAttention(P, list(seqlen), d, B, H, dtype, causal, layout=layout)
+    plan.forward(qd, kd, vd, out, lse)
+    torch.cuda.synchronize()
+    assert bool((out_buf[B * H * S:] == 7.0).all()) and bool((lse_buf[B * H * S:] == 7.0).all())
+    rows = np.arange(w.rows)
+    check_rows(oracle, w, q, k, v, out[:, :, inv].contiguous(), lse[:, :, inv].contiguous(), rows)
+    if layout == "contiguous":
+        # per-step partials against the ring form of the oracle; untouched rows stay untouched
+        _, _, po, pl = oracle.ring_rows(q, k, v, dtype, list(seqlen), rows, causal=causal, tile=32, want_parts=True)
+        for s in range(P):
+            o_part, lse_part = plan.block_forward(s, qd, kd, vd)
+            torch.cuda.synchronize()
+            lg = lse_part.reshape(-1).double().cpu().numpy()
+            active = np.isfinite(pl[:, s])
+            assert np.array_equal(np.isfinite(lg), active)
+            if active.any():
+                assert np.abs(o_part.reshape(-1, d).double().cpu().numpy()[active] - po[active, s]).max() <= 5e-3
+        # the reference-shaped entry, one head, rank by rank
+        q1, k1, v1 = (np.ascontiguousarray(x[0, 0]) for x in (q, k, v))
+        o_ref, _ = oracle.attention_rows(q1[None, None], k1[None, None], v1[None, None], dtype, causal=causal)
+        start = np.concatenate([[0], np.cumsum(seqlen)])
+        for mype in range(P):
+            sl = slice(start[mype], start[mype + 1])
+            o1 = torch.empty((seqlen[mype], d), dtype=qd.dtype, device="cuda")
+            api.ring_attention(to_dev(np.ascontiguousarray(q1[sl]), dtype), to_dev(k1, dtype), to_dev(v1, dtype), o1, P, mype,
+                               list(seqlen), d, max(seqlen), causal=causal)
+            assert np.abs(o1.double().cpu().numpy() - o_ref[sl]).max() <= O_TOL
+    plan.close()
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_grouped_query_heads(oracle, causal):
     # 8 query heads share 2 KV heads: the result equals plain attention with the KV heads repeated
@@ -405,4 +457,4 @@ def test_host_api_checks_on_device():
         plan.forward(x.bfloat16(), x, x)
     plan.close()
     with pytest.raises(api._lib.RingattnError):
-        api.RingAttention(2, 100, 64)                     # chunk not a multiple of 128
+        api.RingAttention(2, 101, 64, causal=True, layout="zigzag")   # the zigzag layout needs even lengths
