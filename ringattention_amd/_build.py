@@ -1,4 +1,5 @@
-"""Builds libringattn.so (HIP kernels + C ABI) in-tree for gfx950 with hipcc."""
+"""Builds libringattn.so (HIP kernels + C ABI) in-tree for gfx950 with hipcc, and the torch
+front end libringattn_torch.so (host code only) with the host compiler."""
 import os
 import shutil
 import subprocess
@@ -7,6 +8,8 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_DIR = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libringattn.so")
+
+TORCH_LIB_PATH = os.path.join(PKG_DIR, "libringattn_torch.so")
 
 SOURCES = ["ringattn_kernels.hip", "ringattn_api.hip", "ringattn_datagen.cpp"]
 
@@ -34,5 +37,33 @@ def build_library(verbose=False):
     return LIB_PATH
 
 
+def build_torch_shim(verbose=False):
+    """Compile csrc/ringattn_torch.cpp (dispatcher op ringattn::fwd on top of the C ABI) against
+    the installed torch.  Host code only; links libringattn.so by relative rpath.  Always recompiles."""
+    import torch
+    from torch.utils import cpp_extension
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if not cxx:
+        raise RuntimeError("g++ not found: cannot build libringattn_torch.so")
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError("build libringattn.so first")
+    tmp = TORCH_LIB_PATH + ".tmp"
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch.compiled_with_cxx11_abi())}"]
+    for inc in cpp_extension.include_paths("cuda") + [os.path.join(REPO_DIR, "include")]:
+        cmd += ["-isystem", inc]
+    cmd += [os.path.join(CSRC, "ringattn_torch.cpp"), "-o", tmp, "-L", torch_lib, "-lc10", "-lc10_hip", "-ltorch_cpu",
+            "-ltorch_hip", "-ltorch", "-L", PKG_DIR, "-l:libringattn.so", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("torch shim build failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
+    if verbose:
+        print(res.stderr)
+    os.replace(tmp, TORCH_LIB_PATH)
+    return TORCH_LIB_PATH
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_torch_shim(verbose=True))
