@@ -232,8 +232,11 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
     return max(0, kv_tail * BN + row - (kv_len - 1)) * ROWB;
   };
   // `checked`: the tile may be kv_tail (steady blocks never issue that one)
+  // A tile index at or beyond n_tiles names a PHANTOM tile: steady blocks run to the end of
+  // the loop and keep loading two blocks ahead; such a load re-reads the last tile into the
+  // ring slot the phantom would use, which no block reads any more.
   auto issue_k = [&](int t, auto checked) {
-    const char* kt = kbase + (int64_t)t * TILE;
+    const char* kt = kbase + (int64_t)min(t, n_tiles - 1) * TILE;
     const unsigned kd = __builtin_amdgcn_readfirstlane(smem_base + (t & (NBUF - 1)) * TILE + wave * (LD * 1024));
     if (decltype(checked)::value && t == kv_tail) {
 #pragma unroll
@@ -244,7 +247,7 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
     }
   };
   auto issue_v = [&](int t, auto checked) {
-    const char* vt = vbase + (int64_t)t * TILE;
+    const char* vt = vbase + (int64_t)min(t, n_tiles - 1) * TILE;
     const unsigned vd = __builtin_amdgcn_readfirstlane(smem_base + (NBUF + (t & (NBUF - 1))) * TILE + wave * (LD * 1024));
     if (decltype(checked)::value && t == kv_tail) {
 #pragma unroll
@@ -271,8 +274,9 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
       for (int qb = 0; qb < QB; ++qb) sacc[qb] = E::mma(kfr, qf[qb][ks], sacc[qb]);
     }
   };
-  auto mask_tile = [&](f32x16(&sacc)[QB], int t) {
-    if (t >= first_masked) {  // key visible iff inside the KV range and key_local <= query_local + diag_off
+  auto mask_tile = [&](f32x16(&sacc)[QB], int t, auto always) {
+    // key visible iff inside the KV range and key_local <= query_local + diag_off
+    if (decltype(always)::value || t >= first_masked) {
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         int lim = kv_len - 1 - t * BN - 4 * h;
@@ -361,9 +365,10 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   // V(u+2), V(u+3), which are issued during this pair.
   // STEADY blocks (all those tiles exist, tiles u+1 and u+2 unmasked) have compile-time ring
   // slots and no conditions.
-  auto block = [&](auto slot_c, auto steady, int u) {
+  auto block = [&](auto slot_c, auto steady, auto masked, int u) {
     constexpr int SLOT = decltype(slot_c)::value;  // u mod 4 (STEADY) or u mod 2 (general)
     constexpr bool STEADY = decltype(steady)::value;
+    constexpr bool MASKED = decltype(masked)::value;  // STEADY only: tile u+1 gets the mask
     f32x16(&cur)[QB] = (SLOT & 1) ? s_odd : s_even;
     f32x16(&nxt)[QB] = (SLOT & 1) ? s_even : s_odd;
     float cand[QB];
@@ -378,6 +383,7 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
         issue_v(u + 1, kUnchecked);
       }
       qk(nxt, (SLOT + 1) & 3);
+      if (MASKED) mask_tile(nxt, u + 1, kChecked);
       exponentials(cur);
       if ((SLOT & 1) == 0) issue_k(u + 4, kUnchecked);
       else issue_v(u + 2, kUnchecked);
@@ -403,7 +409,7 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
       }
       if (u + 1 < n_tiles) {
         qk(nxt, (u + 1) & 3);
-        mask_tile(nxt, u + 1);
+        mask_tile(nxt, u + 1, kUnchecked);
       }
       exponentials(cur);
       pv_product(u & 3);
@@ -425,7 +431,7 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   {
     float cand[QB];
     qk(s_even, 0);
-    mask_tile(s_even, 0);
+    mask_tile(s_even, 0, kUnchecked);
     tile_maxes(s_even, cand);
     move_reference(cand);
   }
@@ -434,20 +440,35 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   using C1 = std::integral_constant<int, 1>;
   using C2 = std::integral_constant<int, 2>;
   using C3 = std::integral_constant<int, 3>;
-  // a steady pair (u, u+1), u even, needs u + 4 < n_tiles (and that tile not to be kv_tail)
-  // and u + 2 < first_masked
-  const int n_steady = min(n_tiles - 4 - (kv_tail >= 0 ? 1 : 0), first_masked - 2);  // pairs starting at u < n_steady
+  // Steady blocks come in groups of four (ring slots are compile-time constants).  A group
+  // starting at u computes the scores of tiles u+1 .. u+4 and loads up to tile u+6:
+  //   plain groups   while those four tiles need no mask; without any mask in the item the last
+  //                  group runs up to tile n_tiles-1 and its last block computes (and drops)
+  //                  the scores of a phantom tile;
+  //   masked groups  (diagonal items) for the rest: every block masks its tile u+1;
+  //   an item with surplus keys in its last tile keeps clear of that tile (its loads need the
+  //   clamped form) and leaves the rest to the general blocks.
+  const bool ragged = kv_tail >= 0;
+  const int plain_end = ragged ? min(first_masked, kv_tail - 2) : (diag ? first_masked : n_tiles + 1);
+  const int masked_end = (diag && !ragged) ? n_tiles + 1 : 0;
   int u = 0;
-  for (; u + 2 < n_steady; u += 4) {
-    block(C0{}, std::true_type{}, u);
-    block(C1{}, std::true_type{}, u + 1);
-    block(C2{}, std::true_type{}, u + 2);
-    block(C3{}, std::true_type{}, u + 3);
+  for (; u + 4 < plain_end; u += 4) {
+    block(C0{}, std::true_type{}, std::false_type{}, u);
+    block(C1{}, std::true_type{}, std::false_type{}, u + 1);
+    block(C2{}, std::true_type{}, std::false_type{}, u + 2);
+    block(C3{}, std::true_type{}, std::false_type{}, u + 3);
+  }
+  for (; u + 4 < masked_end; u += 4) {
+    block(C0{}, std::true_type{}, std::true_type{}, u);
+    block(C1{}, std::true_type{}, std::true_type{}, u + 1);
+    block(C2{}, std::true_type{}, std::true_type{}, u + 2);
+    block(C3{}, std::true_type{}, std::true_type{}, u + 3);
   }
   for (; u < n_tiles; ++u) {
-    if (u & 1) block(C1{}, std::false_type{}, u);
-    else block(C0{}, std::false_type{}, u);
+    if (u & 1) block(C1{}, std::false_type{}, std::false_type{}, u);
+    else block(C0{}, std::false_type{}, std::false_type{}, u);
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // phantom loads may still be in flight
 
   // epilogue (csrc/ring_attention.cu:621-633): normalise, emit partial O and LSE
 #pragma unroll
