@@ -277,12 +277,14 @@ void build_schedule(ringattn_plan* pl) {
 
 int ensure_streams(ringattn_plan* pl) {
   if (pl->streams_ready) return RINGATTN_OK;
+  // a call that failed half way is resumed: nothing is created twice
   const size_t bytes = pl->h_items.size() * sizeof(ringattn::WorkItem);
-  RA_HIP(hipMalloc((void**)&pl->d_items, bytes));
+  if (!pl->d_items) RA_HIP(hipMalloc((void**)&pl->d_items, bytes));
   RA_HIP(hipMemcpy(pl->d_items, pl->h_items.data(), bytes, hipMemcpyHostToDevice));
-  RA_HIP(hipStreamCreateWithFlags(&pl->merge_stream, hipStreamNonBlocking));
-  for (int i = 0; i < kMaxGroups; ++i) RA_HIP(hipEventCreateWithFlags(&pl->ev_group[i], hipEventDisableTiming));
-  RA_HIP(hipEventCreateWithFlags(&pl->ev_done, hipEventDisableTiming));
+  if (!pl->merge_stream) RA_HIP(hipStreamCreateWithFlags(&pl->merge_stream, hipStreamNonBlocking));
+  for (int i = 0; i < kMaxGroups; ++i)
+    if (!pl->ev_group[i]) RA_HIP(hipEventCreateWithFlags(&pl->ev_group[i], hipEventDisableTiming));
+  if (!pl->ev_done) RA_HIP(hipEventCreateWithFlags(&pl->ev_done, hipEventDisableTiming));
   pl->streams_ready = true;
   return RINGATTN_OK;
 }
@@ -425,12 +427,12 @@ int ringattn_plan_destroy(ringattn_plan* plan) {
   int rc = RINGATTN_OK;
   drop_graph(plan);
   if (plan->cap_stream) (void)hipStreamDestroy(plan->cap_stream);
-  if (plan->streams_ready) {
-    (void)hipStreamDestroy(plan->merge_stream);
-    for (int i = 0; i < kMaxGroups; ++i) (void)hipEventDestroy(plan->ev_group[i]);
-    (void)hipEventDestroy(plan->ev_done);
-    (void)hipFree(plan->d_items);
-  }
+  // whatever ensure_streams() got to create, also after a failure half way
+  if (plan->merge_stream) (void)hipStreamDestroy(plan->merge_stream);
+  for (int i = 0; i < kMaxGroups; ++i)
+    if (plan->ev_group[i]) (void)hipEventDestroy(plan->ev_group[i]);
+  if (plan->ev_done) (void)hipEventDestroy(plan->ev_done);
+  if (plan->d_items) (void)hipFree(plan->d_items);
   if (plan->own_ws && plan->ws) {
     hipError_t e = hipFree(plan->ws);
     if (e != hipSuccess) rc = hip_fail(e);

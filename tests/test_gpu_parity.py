@@ -458,3 +458,43 @@ def test_host_api_checks_on_device():
     plan.close()
     with pytest.raises(api._lib.RingattnError):
         api.RingAttention(2, 101, 64, causal=True, layout="zigzag")   # the zigzag layout needs even lengths
+
+
+def test_random_plans_against_oracle(oracle):
+    # seeded sweep over the whole parameter space at small sizes: ranks, ragged lengths, batch,
+    # heads, grouped KV heads, head dim, dtype, mask, layout, explicit scale, graph replay
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        P = int(rng.integers(1, 7))
+        causal = bool(rng.integers(0, 2))
+        zigzag = causal and bool(rng.integers(0, 2))
+        lens = [int(rng.choice([1, 2, 31, 32, 33, 64, 100, 128, 129, 200, 256, 300])) for _ in range(P)]
+        if zigzag:
+            lens = [2 * ((c + 1) // 2) for c in lens]
+        d = int(rng.choice([64, 128]))
+        dtype = str(rng.choice(["fp16", "bf16"]))
+        B, hkv, group = int(rng.integers(1, 3)), int(rng.integers(1, 3)), int(rng.integers(1, 4))
+        H, S = hkv * group, sum(lens)
+        scale = float(rng.choice([0.0, 0.05, 0.2]))
+        graph = bool(rng.integers(0, 2))
+        tag = f"case {case}: P={P} lens={lens} B={B} H={H} hkv={hkv} d={d} {dtype} causal={causal} zigzag={zigzag} scale={scale} graph={graph}"
+        print(tag, flush=True)
+        w = Workload("rand", B, H, d, 1, S, dtype, 1000 + case, causal)
+        q, _, _ = api.make_qkv_bits(w)
+        _, k, v = api.make_qkv_bits(Workload("rand_kv", B, hkv, d, 1, S, dtype, 2000 + case, causal))
+        order = api.zigzag_order(lens) if zigzag else np.arange(S)
+        inv = torch.from_numpy(np.argsort(order)).cuda()
+        qd, kd, vd = (to_dev(np.ascontiguousarray(x[:, :, order]), dtype) for x in (q, k, v))
+        plan = api.RingAttention(P, lens, d, B, H, dtype, causal, softmax_scale=scale, graph=graph,
+                                 kv_heads=hkv if group > 1 else 0, layout="zigzag" if zigzag else "contiguous")
+        out, lse = plan.forward(qd, kd, vd)
+        if graph:                                   # a replay of the captured graph must give the same bits
+            out2, lse2 = plan.forward(qd, kd, vd, torch.empty_like(out), torch.empty_like(lse))
+            out2, lse2 = plan.forward(qd, kd, vd, out2, lse2)
+            torch.cuda.synchronize()
+            assert torch.equal(out, out2) and torch.equal(lse, lse2), tag
+        torch.cuda.synchronize()
+        plan.close()
+        k_full, v_full = (np.repeat(x, group, axis=1) for x in (k, v))
+        check_rows(oracle, w, q, k_full, v_full, out[:, :, inv].contiguous(), lse[:, :, inv].contiguous(),
+                   np.arange(w.rows), scale=scale if scale > 0 else None)
