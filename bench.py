@@ -2,13 +2,14 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4]
 
-A step is one full forward of the workload: the ring step loop (one block-attention
-launch per ring step) plus the P-way merge, with Q/K/V already resident in HBM.  Prints
-one JSON line.  `value` is algorithmic TFLOP/s (4*B*H*d*visible (q,k) pairs per forward)
-over the wall time of K steps; `roofline` prices the block-attention kernel alone
-against the dense MFMA peak, timed with events on the launch stream in a separate
-pass; `merge` does the same for the merge kernel against HBM bandwidth; `cpu_baseline`
-is the CPU oracle timed on this host on a bounded sample of the same workload's rows.
+A step is one full forward of the workload: every ring step of every virtual rank (a few
+block-attention launches) plus the merges of the per-step partials, with Q/K/V already
+resident in HBM.  Prints one JSON line.  `value` is algorithmic TFLOP/s (4*B*H*d*visible
+(q,k) pairs per forward) over the wall time of K steps; `roofline` prices the
+block-attention launches of the same forward against the dense MFMA peak, each timed by an
+event pair on the launch stream (a second pass of K forwards on a plan with the timing
+flag); `merge` times the merge kernel alone against HBM bandwidth; `cpu_baseline` is the
+CPU oracle timed on this host on a bounded sample of the same workload's rows.
 """
 import argparse
 import json
@@ -24,7 +25,7 @@ PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0}
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per block-kernel launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
 # see profiles/; None where not measured for that workload.
-MEASURED_TRAFFIC = {"cfg4": 7.82e8}   # 465.1 MB fetched + 316.9 MB written, average over the 8 launches of a step
+MEASURED_TRAFFIC = {"cfg4": 1.541e9}   # 930.4 MB fetched + 610.7 MB written per launch, average over the 4 launches of a forward
 
 
 def describe(w):
@@ -48,6 +49,7 @@ def main():
     ap.add_argument("--workload", default="cfg4")
     ap.add_argument("--layout", default="contiguous", choices=["contiguous", "zigzag"],
                     help="placement of the sequence on the ranks (zigzag: load-balanced causal ring)")
+    ap.add_argument("--per-step", action="store_true", help="also time one block-attention launch per ring step")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the cpu_baseline sample (0 = skip)")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="only run a plain device copy of MIB mebibytes a few times and exit: the known-size kernel "
@@ -90,44 +92,70 @@ def main():
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     tflops = w.flops / (ms_per_step * 1e-3) / 1e12
 
-    # ---- per-kernel pass: events on the launch stream around each block launch and the merge
-    eager = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=False, layout=args.layout)
-    o_parts = torch.empty((w.npes, w.batch, w.heads, w.seq, w.dim), dtype=torch.float32, device="cuda")
-    l_parts = torch.empty((w.npes, w.batch, w.heads, w.seq), dtype=torch.float32, device="cuda")
-    reps = max(3, min(args.steps, 10))
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(w.npes + 2)] for _ in range(reps)]
-    for rep in range(-1, reps):   # rep -1 warms up
-        for s in range(w.npes):
-            if rep >= 0:
-                ev[rep][s].record(stream)
-            eager.block_forward(s, qd, kd, vd, o_parts[s], l_parts[s], stream)
-        if rep >= 0:
-            ev[rep][w.npes].record(stream)
-        eager.merge_ring(o_parts, l_parts, out, lse, stream)
-        if rep >= 0:
-            ev[rep][w.npes + 1].record(stream)
-    torch.cuda.synchronize()
-    block_ms = [np.mean([ev[r][s].elapsed_time(ev[r][s + 1]) for r in range(reps)]) for s in range(w.npes)]
-    merge_ms = float(np.mean([ev[r][w.npes].elapsed_time(ev[r][w.npes + 1]) for r in range(reps)]))
     bh = w.batch * w.heads
-    launch_flops = [4.0 * w.dim * bh * sum(visible_pairs(it) for it in eager.work_items(s)) for s in range(w.npes)]
-    assert abs(sum(launch_flops) - w.flops) <= 1e-9 * w.flops
-    block_tflops = sum(launch_flops) / (sum(block_ms) * 1e-3) / 1e12
     peak = PEAK_TFLOPS[w.dtype]
+    # ---- block kernel: the same forward on a plan that records an event pair around each of its
+    # block-attention launches, on the stream they are launched on
+    timed = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=False,
+                              layout=args.layout, timing=True)
+    timed.forward(qd, kd, vd, out, lse, stream)
+    launch_ms = []
+    for _ in range(args.steps):
+        timed.forward(qd, kd, vd, out, lse, stream)
+        launch_ms.append(timed.launch_times())
+    launch_ms = np.array(launch_ms)                       # [steps, launches per forward]
+    n_launch = launch_ms.shape[1]
+    avg_launch_ms = float(launch_ms.mean())
+    block_tflops = w.flops / n_launch / (avg_launch_ms * 1e-3) / 1e12
     roofline = {
         "kernel": "block_attention_kernel", "bound": "mfma",
         "achieved": round(block_tflops, 2), "peak": peak, "unit": "TFLOP/s", "frac": round(block_tflops / peak, 4),
         "traffic": MEASURED_TRAFFIC.get(w.name) if args.layout == "contiguous" else None,
-        "launches_per_step": w.npes, "avg_launch_ms": round(float(np.mean(block_ms)), 4),
-        "avg_launch_flop": float(np.mean(launch_flops)),
-        "per_step_ms": [round(float(x), 4) for x in block_ms],
-        "per_step_tflops": [round(f / (t * 1e-3) / 1e12, 1) for f, t in zip(launch_flops, block_ms)],
+        "launches_per_step": n_launch, "avg_launch_ms": round(avg_launch_ms, 4),
+        "avg_launch_flop": w.flops / n_launch,
+        "launch_ms": [round(float(x), 4) for x in launch_ms.mean(axis=0)],
     }
-    # merge: algorithmic bytes = active parts * (4 d + 4) read + (2 d + 4) written, per row
+    timed.close()
+
+    # ---- merge kernel alone: the ring merge on caller-held partials (random numbers: only the
+    # bytes matter), events on the launch stream
+    eager = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=False, layout=args.layout)
+    o_parts = torch.empty((w.npes, w.batch, w.heads, w.seq, w.dim), dtype=torch.float32, device="cuda").normal_()
+    l_parts = torch.empty((w.npes, w.batch, w.heads, w.seq), dtype=torch.float32, device="cuda").normal_()
+    reps = max(3, min(args.steps, 10))
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+    eager.merge_ring(o_parts, l_parts, out, lse, stream)
+    for r in range(reps):
+        ev[r].record(stream)
+        eager.merge_ring(o_parts, l_parts, out, lse, stream)
+    ev[reps].record(stream)
+    torch.cuda.synchronize()
+    merge_ms = float(np.mean([ev[r].elapsed_time(ev[r + 1]) for r in range(reps)]))
+    # algorithmic bytes = active parts * (4 d + 4) read + (2 d + 4) written, per row
     merge_bytes = bh * sum(ln * (bin(act).count("1") * (4 * w.dim + 4) + 2 * w.dim + 4) for _, ln, act in eager.merge_regions())
     merge = {"kernel": "merge_kernel", "bound": "hbm", "achieved": round(merge_bytes / (merge_ms * 1e-3) / 1e9, 1),
              "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(merge_bytes / (merge_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-             "ms": round(merge_ms, 4), "bytes": merge_bytes}
+             "ms": round(merge_ms, 4), "bytes": merge_bytes, "launches": len(eager.merge_regions())}
+
+    # ---- optional: one launch per ring step (what ringattn_block_fwd runs), to show how the work
+    # spreads over the steps of the ring
+    per_step = None
+    if args.per_step:
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(w.npes + 1)] for _ in range(reps)]
+        for rep in range(-1, reps):   # rep -1 warms up
+            for s in range(w.npes):
+                if rep >= 0:
+                    evs[rep][s].record(stream)
+                eager.block_forward(s, qd, kd, vd, o_parts[s], l_parts[s], stream)
+            if rep >= 0:
+                evs[rep][w.npes].record(stream)
+        torch.cuda.synchronize()
+        step_ms = [np.mean([evs[r][s].elapsed_time(evs[r][s + 1]) for r in range(reps)]) for s in range(w.npes)]
+        step_flops = [4.0 * w.dim * bh * sum(visible_pairs(it) for it in eager.work_items(s)) for s in range(w.npes)]
+        assert abs(sum(step_flops) - w.flops) <= 1e-9 * w.flops
+        per_step = {"ms": [round(float(x), 4) for x in step_ms],
+                    "tflops": [round(f / (t * 1e-3) / 1e12, 1) for f, t in zip(step_flops, step_ms)]}
+    del o_parts, l_parts
     eager.close()
     plan.close()
 
@@ -159,7 +187,7 @@ def main():
         "dtype": w.dtype, "data": "synthetic",
         "config": {"workload": describe(w), "algorithmic_flop": w.flops, "graph": bool(w.graph), "layout": args.layout},
         "pct_mfma_peak": round(100.0 * tflops / peak, 2),
-        "roofline": roofline, "merge": merge, "cpu_baseline": cpu,
+        "roofline": roofline, "merge": merge, "per_ring_step": per_step, "cpu_baseline": cpu,
     }))
 
 

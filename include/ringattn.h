@@ -48,6 +48,8 @@ extern "C" {
                                       multiples of this waste no part of a tile */
 
 #define RINGATTN_FLAG_GRAPH 1      /* capture the step loop + merge in a hipGraph and replay it */
+#define RINGATTN_FLAG_TIMING 2     /* record timing events around every block-attention launch of ringattn_fwd
+                                      (read with ringattn_plan_launch_times); ignored together with FLAG_GRAPH */
 
 /*
  * Placement of the sequence on the ranks.  CONTIGUOUS: rank r holds the tokens that follow
@@ -167,6 +169,16 @@ typedef struct ringattn_work_item {
 } ringattn_work_item;
 
 int ringattn_plan_work_items(const ringattn_plan* plan, int step, ringattn_work_item* out, int capacity, int* n_out);
+
+/*
+ * Durations in milliseconds of the block-attention launches of the most recent ringattn_fwd
+ * on a plan created with RINGATTN_FLAG_TIMING, from events recorded on the caller's stream
+ * right before and after each launch -- the job of the cudaEvent pair around the timed loop
+ * of the reference harness (csrc/ring_attention.cu:772-783), per launch.  Blocks until that
+ * forward's launches have finished.  Writes min(n, capacity) values and stores n in *n_out;
+ * RINGATTN_ERR_PLAN if the plan has no timing flag or has not run a forward yet.
+ */
+int ringattn_plan_launch_times(ringattn_plan* plan, float* ms, int capacity, int* n_out);
 
 /*
  * The row ranges ringattn_merge_ring merges separately: rows [start[i], start[i] + len[i])

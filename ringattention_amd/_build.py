@@ -64,6 +64,21 @@ def build_torch_shim(verbose=False):
     return TORCH_LIB_PATH
 
 
+PROBE_PATH = os.path.join(PKG_DIR, "issue_rate_probe")
+
+
+def build_probe():
+    """Compile csrc/issue_rate_probe.hip, the stand-alone instruction-mix micro-benchmark."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    cmd = [hipcc, "--offload-arch=gfx950", "-O2", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           os.path.join(CSRC, "issue_rate_probe.hip"), "-o", PROBE_PATH]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
+    return PROBE_PATH
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_probe())
     print(build_torch_shim(verbose=True))

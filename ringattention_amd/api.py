@@ -17,6 +17,7 @@ from ._lib import RingattnParams, check
 DTYPE_CODE = {"fp16": 0, "bf16": 1, torch.float16: 0, torch.bfloat16: 1}
 TORCH_DTYPE = {0: torch.float16, 1: torch.bfloat16}
 FLAG_GRAPH = 1
+FLAG_TIMING = 2
 LAYOUT_CODE = {"contiguous": 0, "zigzag": 1}
 
 
@@ -53,7 +54,7 @@ class RingAttention:
     """A forward plan for P virtual ring ranks on one GPU."""
 
     def __init__(self, npes, chunk, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, graph=False,
-                 kv_heads=0, layout="contiguous"):
+                 kv_heads=0, layout="contiguous", timing=False):
         """`chunk`: tokens per rank -- one int for equal chunks or a list of npes lengths
         (the per-PE seqlen[] of csrc/ring_attention.cu:753).  `kv_heads`: heads of K and V for
         grouped-query attention (0 = same as `heads`).  `layout`: "contiguous" (rank r holds
@@ -70,7 +71,8 @@ class RingAttention:
         self.seq = sum(self.seqlen)
         self.kv_heads = kv_heads if kv_heads else heads
         self.params = make_params(npes, self.seqlen, dim, batch, heads, dtype, causal, softmax_scale,
-                                  FLAG_GRAPH if graph else 0, kv_heads, LAYOUT_CODE[layout])
+                                  (FLAG_GRAPH if graph else 0) | (FLAG_TIMING if timing else 0), kv_heads,
+                                  LAYOUT_CODE[layout])
         self.handle = ctypes.c_void_p()
         check(self.lib.ringattn_plan_create(ctypes.byref(self.params), None, 0, ctypes.byref(self.handle)),
               "ringattn_plan_create")
@@ -115,6 +117,13 @@ class RingAttention:
         check(self.lib.ringattn_block_fwd(self.handle, int(step), _ptr(q), _ptr(k), _ptr(v), _ptr(o_part),
                                           _ptr(lse_part), _stream_ptr(stream)), "ringattn_block_fwd")
         return o_part, lse_part
+
+    def launch_times(self):
+        """Milliseconds of each block-attention launch of the last forward (plan made with timing=True)."""
+        ms = (ctypes.c_float * 8)()
+        n = ctypes.c_int()
+        check(self.lib.ringattn_plan_launch_times(self.handle, ms, 8, ctypes.byref(n)), "ringattn_plan_launch_times")
+        return [ms[i] for i in range(n.value)]
 
     def work_items(self, step=-1):
         """The plan's block-attention jobs as (q_start, q_len, kv_start, kv_len, diag_off, slot)

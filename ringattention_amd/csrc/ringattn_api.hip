@@ -171,6 +171,8 @@ struct ringattn_plan {
   hipStream_t merge_stream = nullptr;
   hipEvent_t ev_group[kMaxGroups]{};
   hipEvent_t ev_done = nullptr;
+  hipEvent_t ev_t0[kMaxGroups]{}, ev_t1[kMaxGroups]{};  // RINGATTN_FLAG_TIMING: around each block launch
+  bool timed_forward = false;                            // a forward has recorded them
   bool streams_ready = false;
   // hipGraph replay (RINGATTN_FLAG_GRAPH): one captured graph per pointer set
   hipStream_t cap_stream = nullptr;
@@ -285,6 +287,11 @@ int ensure_streams(ringattn_plan* pl) {
   for (int i = 0; i < kMaxGroups; ++i)
     if (!pl->ev_group[i]) RA_HIP(hipEventCreateWithFlags(&pl->ev_group[i], hipEventDisableTiming));
   if (!pl->ev_done) RA_HIP(hipEventCreateWithFlags(&pl->ev_done, hipEventDisableTiming));
+  if (pl->p.flags & RINGATTN_FLAG_TIMING)
+    for (int i = 0; i < kMaxGroups; ++i) {
+      if (!pl->ev_t0[i]) RA_HIP(hipEventCreate(&pl->ev_t0[i]));
+      if (!pl->ev_t1[i]) RA_HIP(hipEventCreate(&pl->ev_t1[i]));
+    }
   pl->streams_ready = true;
   return RINGATTN_OK;
 }
@@ -332,10 +339,13 @@ int run_forward(ringattn_plan* pl, const void* q, const void* k, const void* v, 
                 float* lse, hipStream_t stream) {
   int rc = RINGATTN_OK;
   const size_t G = pl->groups.size();
+  const bool timing = (pl->p.flags & RINGATTN_FLAG_TIMING) && !(pl->p.flags & RINGATTN_FLAG_GRAPH);
   for (size_t g = 0; g < G; ++g) {
     const LaunchGroup& lg = pl->groups[g];
+    if (timing) RA_HIP(hipEventRecord(pl->ev_t0[g], stream));
     rc = launch_items(pl, lg.item_begin, lg.item_count, q, k, v, pl->o_parts, pl->lse_parts, 0, stream);
     if (rc != RINGATTN_OK) return rc;
+    if (timing) RA_HIP(hipEventRecord(pl->ev_t1[g], stream));
     hipStream_t ms = stream;
     if (g + 1 < G) {
       RA_HIP(hipEventRecord(pl->ev_group[g], stream));
@@ -351,6 +361,7 @@ int run_forward(ringattn_plan* pl, const void* q, const void* k, const void* v, 
     RA_HIP(hipEventRecord(pl->ev_done, pl->merge_stream));
     RA_HIP(hipStreamWaitEvent(stream, pl->ev_done, 0));
   }
+  if (timing) pl->timed_forward = true;
   return RINGATTN_OK;
 }
 
@@ -432,6 +443,10 @@ int ringattn_plan_destroy(ringattn_plan* plan) {
   for (int i = 0; i < kMaxGroups; ++i)
     if (plan->ev_group[i]) (void)hipEventDestroy(plan->ev_group[i]);
   if (plan->ev_done) (void)hipEventDestroy(plan->ev_done);
+  for (int i = 0; i < kMaxGroups; ++i) {
+    if (plan->ev_t0[i]) (void)hipEventDestroy(plan->ev_t0[i]);
+    if (plan->ev_t1[i]) (void)hipEventDestroy(plan->ev_t1[i]);
+  }
   if (plan->d_items) (void)hipFree(plan->d_items);
   if (plan->own_ws && plan->ws) {
     hipError_t e = hipFree(plan->ws);
@@ -516,6 +531,19 @@ int ringattn_plan_work_items(const ringattn_plan* plan, int step, ringattn_work_
   for (int i = begin; i < end && i - begin < capacity; ++i) {
     const ringattn::WorkItem& w = plan->h_items[i];
     out[i - begin] = ringattn_work_item{w.q_start, w.q_len, w.kv_start, w.kv_len, w.diag_off, w.slot};
+  }
+  return RINGATTN_OK;
+}
+
+int ringattn_plan_launch_times(ringattn_plan* plan, float* ms, int capacity, int* n_out) {
+  if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
+  if (!n_out || (capacity > 0 && !ms)) return RINGATTN_ERR_NULL;
+  if (!plan->timed_forward) return RINGATTN_ERR_PLAN;
+  const int n = (int)plan->groups.size();
+  *n_out = n;
+  for (int g = 0; g < n && g < capacity; ++g) {
+    RA_HIP(hipEventSynchronize(plan->ev_t1[g]));
+    RA_HIP(hipEventElapsedTime(&ms[g], plan->ev_t0[g], plan->ev_t1[g]));
   }
   return RINGATTN_OK;
 }

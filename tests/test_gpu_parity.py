@@ -498,3 +498,23 @@ def test_random_plans_against_oracle(oracle):
         k_full, v_full = (np.repeat(x, group, axis=1) for x in (k, v))
         check_rows(oracle, w, q, k_full, v_full, out[:, :, inv].contiguous(), lse[:, :, inv].contiguous(),
                    np.arange(w.rows), scale=scale if scale > 0 else None)
+
+
+def test_launch_times_of_a_timed_plan():
+    w = Workload("timed", 1, 4, 128, 8, 256, "bf16", 97, True)
+    q, k, v = (to_dev(x, w.dtype) for x in api.make_qkv_bits(w))
+    plain = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, True)
+    o_ref, l_ref = plain.forward(q, k, v)
+    with pytest.raises(api._lib.RingattnError):
+        plain.launch_times()                                  # no timing flag
+    plain.close()
+    timed = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, True, timing=True)
+    with pytest.raises(api._lib.RingattnError):
+        timed.launch_times()                                  # no forward yet
+    out, lse = timed.forward(q, k, v)
+    ms = timed.launch_times()
+    torch.cuda.synchronize()
+    n_items = len(timed.work_items(-1))
+    assert 1 <= len(ms) <= 8 and n_items == 36 and all(0.0 < t < 1000.0 for t in ms)
+    assert torch.equal(out, o_ref) and torch.equal(lse, l_ref)    # the flag changes nothing in the result
+    timed.close()
