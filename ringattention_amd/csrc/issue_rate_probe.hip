@@ -23,6 +23,8 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 #define FMA(x) asm volatile("v_fma_f32 %0, %0, %0, %0" : "+v"(x))
 #define EXP(x) asm volatile("v_exp_f32 %0, %0" : "+v"(x))
 
+constexpr int kRepeat = 8;  // groups of 4 MFMAs per loop iteration: the loop overhead must not count
+
 enum Mix { kMfma, kMfmaValu, kMfmaValuLds, kMfmaValuHalfLds, kExp, kFma, kCvt, kMax3, kReadB128, kReadTr };
 
 template <int MIX>
@@ -38,8 +40,8 @@ __global__ __launch_bounds__(512) void probe(long long* ticks, float* sink, int 
     a[i] = (__bf16)(seed + i);
     b[i] = (__bf16)(seed - i);
   }
-  f32x4 q0, q1, q2, q3;
-  f32x2 h0, h1, h2, h3;
+  f32x4 q0 = {0}, q1 = {0}, q2, q3;
+  f32x2 h0 = {0}, h1 = {0}, h2 = {0}, h3 = {0};
   const unsigned wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const unsigned base = (unsigned)(uintptr_t)(const __attribute__((address_space(3))) void*)lds + (wave & 3) * 8192;
   const unsigned addr16 = base + lane * 16, addr8 = base + lane * 8;  // conflict-free
@@ -47,30 +49,34 @@ __global__ __launch_bounds__(512) void probe(long long* ticks, float* sink, int 
   const long long t0 = clock64();
   for (int it = 0; it < iters; ++it) {
     if (MIX == kMfma) {
-      MFMA(acc0); MFMA(acc1); MFMA(acc0); MFMA(acc1);
+#pragma unroll
+      for (int r = 0; r < kRepeat; ++r) {
+        MFMA(acc0); MFMA(acc1); MFMA(acc0); MFMA(acc1);
+      }
     } else if (MIX == kMfmaValu || MIX == kMfmaValuLds || MIX == kMfmaValuHalfLds) {
-      // per MFMA: 4 plain VALU ops and one exponential; per 4 MFMAs 4 KB (or 2 KB) of fragments
-      if (MIX == kMfmaValuLds) {
-        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024" : "=v"(q0), "=v"(q1) : "v"(addr16));
-        asm volatile("ds_read_b64_tr_b16 %0, %4\n\tds_read_b64_tr_b16 %1, %4 offset:512\n\t"
-                     "ds_read_b64_tr_b16 %2, %4 offset:1024\n\tds_read_b64_tr_b16 %3, %4 offset:1536"
-                     : "=v"(h0), "=v"(h1), "=v"(h2), "=v"(h3) : "v"(addr8));
-      } else if (MIX == kMfmaValuHalfLds) {
-        asm volatile("ds_read_b128 %0, %1" : "=v"(q0) : "v"(addr16));
-        asm volatile("ds_read_b64_tr_b16 %0, %2\n\tds_read_b64_tr_b16 %1, %2 offset:512" : "=v"(h0), "=v"(h1) : "v"(addr8));
-      }
+      // per MFMA: 4 plain VALU ops and one exponential; per 4 MFMAs 4 KB (or 2 KB) of fragments,
+      // read one group of four MFMAs ahead of the wait
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        if (g & 1) MFMA(acc1);
-        else MFMA(acc0);
+      for (int r = 0; r < kRepeat; ++r) {
+        if (MIX == kMfmaValuLds) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::"v"(q0), "v"(q1), "v"(h0), "v"(h1), "v"(h2), "v"(h3) : "memory");
+          asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024" : "=v"(q0), "=v"(q1) : "v"(addr16));
+          asm volatile("ds_read_b64_tr_b16 %0, %4\n\tds_read_b64_tr_b16 %1, %4 offset:512\n\t"
+                       "ds_read_b64_tr_b16 %2, %4 offset:1024\n\tds_read_b64_tr_b16 %3, %4 offset:1536"
+                       : "=v"(h0), "=v"(h1), "=v"(h2), "=v"(h3) : "v"(addr8));
+        } else if (MIX == kMfmaValuHalfLds) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::"v"(q0), "v"(h0), "v"(h1) : "memory");
+          asm volatile("ds_read_b128 %0, %1" : "=v"(q0) : "v"(addr16));
+          asm volatile("ds_read_b64_tr_b16 %0, %2\n\tds_read_b64_tr_b16 %1, %2 offset:512" : "=v"(h0), "=v"(h1) : "v"(addr8));
+        }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) FMA(x[4 * g + i]);
-        EXP(x[4 * g]);
-      }
-      if (MIX == kMfmaValuLds) {
-        asm volatile("s_waitcnt lgkmcnt(0)" ::"v"(q0), "v"(q1), "v"(h0), "v"(h1), "v"(h2), "v"(h3) : "memory");
-      } else if (MIX == kMfmaValuHalfLds) {
-        asm volatile("s_waitcnt lgkmcnt(0)" ::"v"(q0), "v"(h0), "v"(h1) : "memory");
+        for (int g = 0; g < 4; ++g) {
+          if (g & 1) MFMA(acc1);
+          else MFMA(acc0);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) FMA(x[4 * g + i]);
+          EXP(x[4 * g]);
+        }
       }
     } else if (MIX == kExp) {
 #pragma unroll
@@ -122,15 +128,15 @@ double run(int iters) {
 }
 
 int main(int argc, char** argv) {
-  const int iters = argc > 1 ? atoi(argv[1]) : 20000;
-  const double mfma = run<kMfma>(iters);  // 4 MFMAs per wave, 8 per SIMD and iteration
-  printf("two waves per SIMD, %d iterations; ticks = s_memtime counts per iteration and wave\n", iters);
+  const int iters = argc > 1 ? atoi(argv[1]) : 5000;
+  const double mfma = run<kMfma>(iters) / kRepeat;  // 4 MFMAs per wave, 8 per SIMD
+  printf("two waves per SIMD, %d iterations; ticks = s_memtime counts per group of 4 MFMAs and wave\n", iters);
   printf("%-58s %8.1f ticks  MFMA utilisation 100.0 %%\n", "4 mfma_f32_32x32x16_bf16", mfma);
-  const double v = run<kMfmaValu>(iters);
+  const double v = run<kMfmaValu>(iters) / kRepeat;
   printf("%-58s %8.1f ticks  MFMA utilisation %5.1f %%\n", "4 mfma + 16 v_fma_f32 + 4 v_exp_f32", v, 100 * mfma / v);
-  const double l = run<kMfmaValuLds>(iters);
+  const double l = run<kMfmaValuLds>(iters) / kRepeat;
   printf("%-58s %8.1f ticks  MFMA utilisation %5.1f %%\n", "  + 2 ds_read_b128 + 4 ds_read_b64_tr_b16 (4 KB)", l, 100 * mfma / l);
-  const double hl = run<kMfmaValuHalfLds>(iters);
+  const double hl = run<kMfmaValuHalfLds>(iters) / kRepeat;
   printf("%-58s %8.1f ticks  MFMA utilisation %5.1f %%\n", "  + 1 ds_read_b128 + 2 ds_read_b64_tr_b16 (2 KB)", hl, 100 * mfma / hl);
   const double per_mfma = mfma / 8.0;  // ticks of one MFMA (32 cycles) when the pipe is saturated
   printf("single instruction classes, cycles per instruction and wave (one MFMA = 32 cycles):\n");
