@@ -518,3 +518,13 @@ def test_launch_times_of_a_timed_plan():
     assert 1 <= len(ms) <= 8 and n_items == 36 and all(0.0 < t < 1000.0 for t in ms)
     assert torch.equal(out, o_ref) and torch.equal(lse, l_ref)    # the flag changes nothing in the result
     timed.close()
+
+
+def test_maximum_ranks_long_sequence(oracle):
+    # the largest ring the ABI takes (64 ranks) at a real chunk size: S = 262 144 tokens, one head;
+    # 64 partial slots of 135 MB, 2 080 work items; rows sampled (first rows, chunk edges, random)
+    w = Workload("max_ring", 1, 1, 128, 64, 4096, "bf16", 99, True)
+    q, k, v = api.make_qkv_bits(w)
+    out, lse = forward(w, q, k, v)
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    check_rows(oracle, w, q, k, v, out, lse, sample_rows(w, 192))
