@@ -77,7 +77,8 @@ def main():
 
     q, k, v = api.make_qkv_bits(w)
     qd, kd, vd = (api.bits_to_tensor(x, w.dtype) for x in (q, k, v))
-    plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=w.graph, layout=args.layout)
+    plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=w.graph, layout=args.layout,
+                             half_partials=w.half_partials)
     out = torch.empty_like(qd)
     lse = torch.empty((w.batch, w.heads, w.seq), dtype=torch.float32, device="cuda")
     stream = torch.cuda.current_stream()
@@ -97,7 +98,7 @@ def main():
     # ---- block kernel: the same forward on a plan that records an event pair around each of its
     # block-attention launches, on the stream they are launched on
     timed = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=False,
-                              layout=args.layout, timing=True)
+                              layout=args.layout, timing=True, half_partials=w.half_partials)
     timed.forward(qd, kd, vd, out, lse, stream)
     launch_ms = []
     for _ in range(args.steps):
@@ -119,8 +120,9 @@ def main():
 
     # ---- merge kernel alone: the ring merge on caller-held partials (random numbers: only the
     # bytes matter), events on the launch stream
-    eager = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=False, layout=args.layout)
-    o_parts = torch.empty((w.npes, w.batch, w.heads, w.seq, w.dim), dtype=torch.float32, device="cuda").normal_()
+    eager = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=False, layout=args.layout,
+                              half_partials=w.half_partials)
+    o_parts = torch.empty((w.npes, w.batch, w.heads, w.seq, w.dim), dtype=eager.part_dtype, device="cuda").normal_()
     l_parts = torch.empty((w.npes, w.batch, w.heads, w.seq), dtype=torch.float32, device="cuda").normal_()
     reps = max(3, min(args.steps, 10))
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
@@ -131,8 +133,9 @@ def main():
     ev[reps].record(stream)
     torch.cuda.synchronize()
     merge_ms = float(np.mean([ev[r].elapsed_time(ev[r + 1]) for r in range(reps)]))
-    # algorithmic bytes = active parts * (4 d + 4) read + (2 d + 4) written, per row
-    merge_bytes = bh * sum(ln * (bin(act).count("1") * (4 * w.dim + 4) + 2 * w.dim + 4) for _, ln, act in eager.merge_regions())
+    # algorithmic bytes = active parts * (4 d + 4) read (2 d + 4 with fp16 partials) + (2 d + 4) written, per row
+    part_row = (2 if w.half_partials else 4) * w.dim + 4
+    merge_bytes = bh * sum(ln * (bin(act).count("1") * part_row + 2 * w.dim + 4) for _, ln, act in eager.merge_regions())
     merge = {"kernel": "merge_kernel", "bound": "hbm", "achieved": round(merge_bytes / (merge_ms * 1e-3) / 1e9, 1),
              "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(merge_bytes / (merge_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
              "ms": round(merge_ms, 4), "bytes": merge_bytes, "launches": len(eager.merge_regions())}
@@ -185,7 +188,8 @@ def main():
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w.dtype, "data": "synthetic",
-        "config": {"workload": describe(w), "algorithmic_flop": w.flops, "graph": bool(w.graph), "layout": args.layout},
+        "config": {"workload": describe(w), "algorithmic_flop": w.flops, "graph": bool(w.graph), "layout": args.layout,
+                   "partials": "fp16" if w.half_partials else "fp32"},
         "pct_mfma_peak": round(100.0 * tflops / peak, 2),
         "roofline": roofline, "merge": merge, "per_ring_step": per_step, "cpu_baseline": cpu,
     }))

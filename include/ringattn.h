@@ -50,6 +50,10 @@ extern "C" {
 #define RINGATTN_FLAG_GRAPH 1      /* capture the step loop + merge in a hipGraph and replay it */
 #define RINGATTN_FLAG_TIMING 2     /* record timing events around every block-attention launch of ringattn_fwd
                                       (read with ringattn_plan_launch_times); ignored together with FLAG_GRAPH */
+#define RINGATTN_FLAG_HALF_PARTIALS 4 /* keep the per-step partial O in fp16 instead of fp32 (for either input dtype): halves
+                                      the workspace and the bytes the block kernel writes and the merge reads.  A partial O
+                                      row is a weighted mean of V rows, so this needs |V| < 65504, and it adds up to 2^-11
+                                      relative error per partial (fp32 partials add none); the partial LSE stays fp32 */
 
 /*
  * Placement of the sequence on the ranks.  CONTIGUOUS: rank r holds the tokens that follow
@@ -91,7 +95,8 @@ typedef struct ringattn_params {
 typedef struct ringattn_plan ringattn_plan;
 
 /* Bytes of device workspace a plan needs (per-step partial O and LSE for every ring
- * step): npes * batch*heads*S * (dim + 1) * 4.  0 if the parameters are invalid. */
+ * step): npes * batch*heads*S * (dim + 1) * 4, or npes * batch*heads*S * (2 dim + 4) with
+ * RINGATTN_FLAG_HALF_PARTIALS.  0 if the parameters are invalid. */
 size_t ringattn_workspace_bytes(const ringattn_params* params);
 
 /*
@@ -124,13 +129,14 @@ int ringattn_fwd(ringattn_plan* plan, const void* q, const void* k, const void* 
 /*
  * One ring step (the body of the reference's step loop, csrc/ring_attention.cu:456-620,
  * for every active rank at once): rank r attends KV chunk (r + step) mod npes and the
- * normalised fp32 partial O [batch, heads, S, dim] and fp32 partial LSE
+ * normalised partial O [batch, heads, S, dim] (fp32; fp16 on a plan with
+ * RINGATTN_FLAG_HALF_PARTIALS) and fp32 partial LSE
  * [batch, heads, S] are written for the rows of the active ranks.  Rows that see no key of
  * the visited chunk (causal: chunk j > r; zigzag: also the low half against j > r) are
  * left untouched.
  */
 int ringattn_block_fwd(ringattn_plan* plan, int step, const void* q, const void* k, const void* v,
-                       float* o_part, float* lse_part, void* stream);
+                       void* o_part, float* lse_part, void* stream);
 
 /*
  * Cross-step merge (no function of its own in the reference: it is the algebra of
@@ -150,7 +156,7 @@ int ringattn_merge(const float* o_parts, const float* lse_parts, int n_parts, in
  * r + s >= npes for a row of rank r), so parts the step loop never wrote are never touched.  Like ringattn_merge, it has no counterpart
  * function in the reference (csrc/ring_attention.cu:207-245,621-633 pin the algebra).
  */
-int ringattn_merge_ring(ringattn_plan* plan, const float* o_parts, const float* lse_parts,
+int ringattn_merge_ring(ringattn_plan* plan, const void* o_parts, const float* lse_parts,
                         void* out, float* lse, void* stream);
 
 /*

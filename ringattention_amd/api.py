@@ -18,6 +18,7 @@ DTYPE_CODE = {"fp16": 0, "bf16": 1, torch.float16: 0, torch.bfloat16: 1}
 TORCH_DTYPE = {0: torch.float16, 1: torch.bfloat16}
 FLAG_GRAPH = 1
 FLAG_TIMING = 2
+FLAG_HALF_PARTIALS = 4
 LAYOUT_CODE = {"contiguous": 0, "zigzag": 1}
 
 
@@ -54,12 +55,13 @@ class RingAttention:
     """A forward plan for P virtual ring ranks on one GPU."""
 
     def __init__(self, npes, chunk, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, graph=False,
-                 kv_heads=0, layout="contiguous", timing=False):
+                 kv_heads=0, layout="contiguous", timing=False, half_partials=False):
         """`chunk`: tokens per rank -- one int for equal chunks or a list of npes lengths
         (the per-PE seqlen[] of csrc/ring_attention.cu:753).  `kv_heads`: heads of K and V for
         grouped-query attention (0 = same as `heads`).  `layout`: "contiguous" (rank r holds
         the tokens after those of rank r-1) or "zigzag" (rank r holds a low and a high
-        half-chunk; see zigzag_order)."""
+        half-chunk; see zigzag_order).  `half_partials`: keep the per-step partial O in fp16
+        (half the workspace and merge traffic; needs |V| < 65504)."""
         self.lib = _lib.load()
         self.seqlen = [int(chunk)] * npes if isinstance(chunk, int) else [int(x) for x in chunk]
         if len(self.seqlen) != npes:
@@ -68,10 +70,12 @@ class RingAttention:
         self.dtype_code = DTYPE_CODE[dtype]
         self.torch_dtype = TORCH_DTYPE[self.dtype_code]
         self.causal = bool(causal)
+        self.part_dtype = torch.float16 if half_partials else torch.float32
         self.seq = sum(self.seqlen)
         self.kv_heads = kv_heads if kv_heads else heads
         self.params = make_params(npes, self.seqlen, dim, batch, heads, dtype, causal, softmax_scale,
-                                  (FLAG_GRAPH if graph else 0) | (FLAG_TIMING if timing else 0), kv_heads,
+                                  (FLAG_GRAPH if graph else 0) | (FLAG_TIMING if timing else 0)
+                                  | (FLAG_HALF_PARTIALS if half_partials else 0), kv_heads,
                                   LAYOUT_CODE[layout])
         self.handle = ctypes.c_void_p()
         check(self.lib.ringattn_plan_create(ctypes.byref(self.params), None, 0, ctypes.byref(self.handle)),
@@ -111,7 +115,8 @@ class RingAttention:
         for t, nm in ((q, "q"), (k, "k"), (v, "v")):
             _check_tensor(t, nm, self.torch_dtype)
         if o_part is None:
-            o_part = torch.zeros(self._shape(), dtype=torch.float32, device=q.device)
+            o_part = torch.zeros(self._shape(), dtype=self.part_dtype, device=q.device)
+        _check_tensor(o_part, "o_part", self.part_dtype)
         if lse_part is None:
             lse_part = torch.full((self.batch, self.heads, self.seq), float("-inf"), dtype=torch.float32, device=q.device)
         check(self.lib.ringattn_block_fwd(self.handle, int(step), _ptr(q), _ptr(k), _ptr(v), _ptr(o_part),
@@ -146,7 +151,7 @@ class RingAttention:
 
     def merge_ring(self, o_parts, lse_parts, out=None, lse=None, stream=None):
         """Ring-aware merge of caller-held per-step partials [npes, B, H, S, d] / [npes, B, H, S]."""
-        _check_tensor(o_parts, "o_parts", torch.float32)
+        _check_tensor(o_parts, "o_parts", self.part_dtype)
         _check_tensor(lse_parts, "lse_parts", torch.float32)
         if out is None:
             out = torch.empty(self._shape(), dtype=self.torch_dtype, device=o_parts.device)

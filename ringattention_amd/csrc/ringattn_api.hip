@@ -90,8 +90,12 @@ int validate(const ringattn_params* p, Derived* d) {
 
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
+inline bool half_partials(const ringattn_params& p) { return (p.flags & RINGATTN_FLAG_HALF_PARTIALS) != 0; }
+
+// partial O of every slot (fp32, or fp16 with RINGATTN_FLAG_HALF_PARTIALS), then the fp32 partial LSEs
 size_t workspace_bytes_of(const ringattn_params* p, const Derived& d) {
-  return (size_t)p->npes * (size_t)d.rows * (size_t)(p->dim + 1) * sizeof(float);
+  const size_t o_elem = half_partials(*p) ? 2 : 4;
+  return (size_t)p->npes * (size_t)d.rows * ((size_t)p->dim * o_elem + sizeof(float));
 }
 
 inline ringattn::WorkItem make_item(int q_start, int q_len, int kv_start, int kv_len, int diag_off, int slot) {
@@ -153,7 +157,7 @@ struct ringattn_plan {
   void* ws = nullptr;
   size_t ws_bytes = 0;
   bool own_ws = false;
-  float* o_parts = nullptr;    // [npes, rows, dim]
+  void* o_parts = nullptr;     // [npes, rows, dim] fp32 (fp16 with RINGATTN_FLAG_HALF_PARTIALS)
   float* lse_parts = nullptr;  // [npes, rows]
   // Item table (host copy + device copy made at the first forward): first the launch
   // schedule of ringattn_fwd, then one list per ring step for ringattn_block_fwd.
@@ -196,6 +200,7 @@ void fill_geometry(ringattn::BlockStepArgs& a, const ringattn_params& p, const D
   a.heads = p.heads;
   a.kv_group = p.kv_heads > 0 ? p.heads / p.kv_heads : 1;
   a.scale_log2 = d.scale * kLog2e;
+  a.half_partials = half_partials(p) ? 1 : 0;
 }
 
 // The rows of rank r that share a set of active slots, with that set: slot s is active for
@@ -298,7 +303,7 @@ int ensure_streams(ringattn_plan* pl) {
 
 // A block launch over a slice of the item table; o_part / lse_part: partial slot `slot_bias`.
 int launch_items(const ringattn_plan* pl, int item_begin, int item_count, const void* q, const void* k,
-                 const void* v, float* o_part, float* lse_part, int slot_bias, hipStream_t stream) {
+                 const void* v, void* o_part, float* lse_part, int slot_bias, hipStream_t stream) {
   ringattn::BlockStepArgs a;
   fill_geometry(a, pl->p, pl->d);
   a.q = q;
@@ -314,7 +319,7 @@ int launch_items(const ringattn_plan* pl, int item_begin, int item_count, const 
   return RINGATTN_OK;
 }
 
-int launch_region_merge(const ringattn_plan* pl, const float* o_parts, const float* lse_parts, void* out,
+int launch_region_merge(const ringattn_plan* pl, const void* o_parts, const float* lse_parts, void* out,
                         float* lse, hipStream_t stream, const MergeRegion& reg) {
   ringattn::MergeArgs m;
   m.o_parts = o_parts;
@@ -326,6 +331,7 @@ int launch_region_merge(const ringattn_plan* pl, const float* o_parts, const flo
   m.rows = pl->d.BH * reg.len;
   m.part_stride_rows = pl->d.rows;
   m.active = reg.active;
+  m.half_partials = half_partials(pl->p) ? 1 : 0;
   m.S = (int)pl->d.S;
   RA_HIP(ringattn::launch_merge(m, pl->p.dtype, pl->p.dim, stream));
   return RINGATTN_OK;
@@ -419,8 +425,8 @@ int ringattn_plan_create(const ringattn_params* params, void* workspace, size_t 
     }
     pl->own_ws = true;
   }
-  pl->o_parts = (float*)pl->ws;
-  pl->lse_parts = pl->o_parts + (size_t)params->npes * d.rows * params->dim;
+  pl->o_parts = pl->ws;
+  pl->lse_parts = (float*)((char*)pl->ws + (size_t)params->npes * d.rows * params->dim * (half_partials(*params) ? 2 : 4));
   build_schedule(pl);
   {
     std::lock_guard<std::mutex> lk(g_plans_mu);
@@ -498,7 +504,7 @@ int ringattn_fwd(ringattn_plan* plan, const void* q, const void* k, const void* 
 }
 
 int ringattn_block_fwd(ringattn_plan* plan, int step, const void* q, const void* k, const void* v,
-                       float* o_part, float* lse_part, void* stream) {
+                       void* o_part, float* lse_part, void* stream) {
   if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
   if (!q || !k || !v || !o_part || !lse_part) return RINGATTN_ERR_NULL;
   if (step < 0 || step >= plan->p.npes) return RINGATTN_ERR_RANK;
@@ -509,7 +515,7 @@ int ringattn_block_fwd(ringattn_plan* plan, int step, const void* q, const void*
                       o_part, lse_part, step, (hipStream_t)stream);
 }
 
-int ringattn_merge_ring(ringattn_plan* plan, const float* o_parts, const float* lse_parts, void* out,
+int ringattn_merge_ring(ringattn_plan* plan, const void* o_parts, const float* lse_parts, void* out,
                         float* lse, void* stream) {
   if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
   if (!o_parts || !lse_parts || !out || !lse) return RINGATTN_ERR_NULL;
@@ -578,6 +584,7 @@ int ringattn_merge(const float* o_parts, const float* lse_parts, int n_parts, in
   m.rows = rows;
   m.part_stride_rows = rows;
   m.active = n_parts >= 64 ? ~(uint64_t)0 : (((uint64_t)1 << n_parts) - 1);
+  m.half_partials = 0;
   m.S = (int)(rows > 0 ? (rows < INT32_MAX ? rows : INT32_MAX) : 1);
   m.sel_start = 0;
   m.sel_len = m.S;

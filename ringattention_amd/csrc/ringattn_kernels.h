@@ -30,7 +30,7 @@ struct BlockStepArgs {
   const void* q;       // [BH, S, D] storage dtype
   const void* k;       // [batch * heads / kv_group, S, D]
   const void* v;       // [batch * heads / kv_group, S, D]
-  float* o_part;       // partial slot `slot_bias`: [BH, S, D] fp32 partial O (normalised)
+  void* o_part;        // partial slot `slot_bias`: [BH, S, D] partial O (normalised), fp32 or fp16 (half_partials)
   float* lse_part;     // partial slot `slot_bias`: [BH, S] fp32 partial LSE (natural log)
   const WorkItem* items;     // device array
   int64_t bh_stride;   // elements between heads of q (= S * D)
@@ -44,12 +44,13 @@ struct BlockStepArgs {
   int heads;           // query heads per batch entry
   int kv_group;        // query heads per KV head (1 = one KV head per query head)
   float scale_log2;    // softmax_scale * log2(e)
+  int half_partials;   // partial O stored as fp16 instead of fp32
 };
 
 // Merge of (O, LSE) partials into the final O (storage dtype) and LSE, for the rows
 // [sel_start, sel_start + sel_len) of every head.
 struct MergeArgs {
-  const float* o_parts;   // [slots, heads * S, D]
+  const void* o_parts;    // [slots, heads * S, D] fp32, or fp16 with half_partials
   const float* lse_parts; // [slots, heads * S]
   void* out;              // [heads * S, D] storage dtype
   float* lse;             // [heads * S]
@@ -58,6 +59,7 @@ struct MergeArgs {
   uint64_t active;        // bit s set: slot s holds a partial for these rows; other slots are never read
   int S;                  // rows per head
   int sel_start, sel_len; // row range within a head
+  int half_partials;
 };
 
 // dtype: 0 = fp16, 1 = bf16.  Return hipSuccess or the launch error.

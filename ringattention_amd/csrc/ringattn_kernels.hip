@@ -37,6 +37,7 @@ namespace ringattn {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -116,7 +117,7 @@ template <int D> static __device__ __forceinline__ int v_swizzle(int row) {
 // branches.  Until then p = exp2((s - m) k2) may exceed 1 (by at most 2^kLazyLog2, well
 // inside fp16 and bf16 range); O = acc / l and LSE = (m k2 + log2 l) ln 2 do not depend on
 // the choice of m.
-template <int DT, int D>
+template <int DT, int D, bool HP>
 __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStepArgs a) {
   using E = Elem<DT>;
   constexpr int QB = 1;            // 32-query blocks per wave
@@ -479,7 +480,7 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
     if (row_l >= q_len) continue;  // a row beyond the query range
     const int row_g = q_start + row_l;
     const int64_t slot_rows = (int64_t)(w.slot - a.slot_bias) * a.part_stride_rows;
-    float* orow = a.o_part + (slot_rows + (int64_t)bh * a.S + row_g) * D;
+    const int64_t opos = (slot_rows + (int64_t)bh * a.S + row_g) * D;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -487,7 +488,14 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
         f32x4 val;
 #pragma unroll
         for (int e = 0; e < 4; ++e) val[e] = oacc[qb][db][4 * q4 + e] * inv;
-        *(f32x4*)(orow + 32 * db + 8 * q4 + 4 * h) = val;
+        if (HP) {  // fp16 partials: |O_part| <= max |V|, the caller vouches that this fits
+          f16x4 hv;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) hv[e] = (_Float16)val[e];
+          *(f16x4*)((_Float16*)a.o_part + opos + 32 * db + 8 * q4 + 4 * h) = hv;
+        } else {
+          *(f32x4*)((float*)a.o_part + opos + 32 * db + 8 * q4 + 4 * h) = val;
+        }
       }
     if (h == 0) {
       const float lse = (l > 0.f) ? (ms[qb] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
@@ -515,7 +523,28 @@ template <> struct Store8<1> {
   }
 };
 
-template <int DT, int D>
+// 8 consecutive columns of one partial row as floats
+template <bool HP> struct PartRow;
+template <> struct PartRow<false> {
+  using ptr = const float*;
+  static __device__ __forceinline__ void ld(ptr p, f32x4& x0, f32x4& x1) {
+    x0 = *(const f32x4*)p;
+    x1 = *(const f32x4*)(p + 4);
+  }
+};
+template <> struct PartRow<true> {
+  using ptr = const _Float16*;
+  static __device__ __forceinline__ void ld(ptr p, f32x4& x0, f32x4& x1) {
+    const f16x8 v = *(const f16x8*)p;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      x0[e] = (float)v[e];
+      x1[e] = (float)v[4 + e];
+    }
+  }
+};
+
+template <int DT, int D, bool HP>
 __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
   constexpr int TPR = D / 8;  // threads per row, 8 columns each
   constexpr int ROWS = 256 / TPR;
@@ -525,7 +554,7 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
   const int c8 = threadIdx.x % TPR;
   // active slots of these rows: the set bits of a.active, visited in ascending order
   const float* lse_row = a.lse_parts + row;
-  const float* o_row = a.o_parts + row * D + c8 * 8;
+  const typename PartRow<HP>::ptr o_row = (typename PartRow<HP>::ptr)a.o_parts + row * D + c8 * 8;
   const int64_t lse_stride = a.part_stride_rows, o_stride = a.part_stride_rows * D;
 
   float mx = -INFINITY;
@@ -545,8 +574,7 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
         const int64_t s = __builtin_ctzll(rest);
         rest &= rest - 1;
         L[u] = lse_row[s * lse_stride];
-        x0[u] = *(const f32x4*)(o_row + s * o_stride);
-        x1[u] = *(const f32x4*)(o_row + s * o_stride + 4);
+        PartRow<HP>::ld(o_row + s * o_stride, x0[u], x1[u]);
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
@@ -564,7 +592,8 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
       const int64_t s = __builtin_ctzll(rest);
       const float Ls = lse_row[s * lse_stride];
       const float w = __expf(Ls - mx);
-      const f32x4 x0 = *(const f32x4*)(o_row + s * o_stride), x1 = *(const f32x4*)(o_row + s * o_stride + 4);
+      f32x4 x0, x1;
+      PartRow<HP>::ld(o_row + s * o_stride, x0, x1);
       if (Ls == -INFINITY) continue;
       wsum += w;
 #pragma unroll
@@ -589,10 +618,16 @@ hipError_t launch_block_step(const BlockStepArgs& a, int dtype, int dim, hipStre
   const int64_t blocks = ((groups + 7) / 8) * 8 * q_tiles;
   if (q_tiles <= 0 || blocks > INT32_MAX) return hipErrorInvalidValue;
   const unsigned grid = (unsigned)blocks;
-  if (dtype == 0 && dim == 64) block_attention_kernel<0, 64><<<grid, 256, 0, stream>>>(a);
-  else if (dtype == 0 && dim == 128) block_attention_kernel<0, 128><<<grid, 256, 0, stream>>>(a);
-  else if (dtype == 1 && dim == 64) block_attention_kernel<1, 64><<<grid, 256, 0, stream>>>(a);
-  else if (dtype == 1 && dim == 128) block_attention_kernel<1, 128><<<grid, 256, 0, stream>>>(a);
+#define RA_LAUNCH_BLOCK(DT_, D_)                                                            \
+  do {                                                                                   \
+    if (a.half_partials) block_attention_kernel<DT_, D_, true><<<grid, 256, 0, stream>>>(a);  \
+    else block_attention_kernel<DT_, D_, false><<<grid, 256, 0, stream>>>(a);                \
+  } while (0)
+  if (dtype == 0 && dim == 64) RA_LAUNCH_BLOCK(0, 64);
+  else if (dtype == 0 && dim == 128) RA_LAUNCH_BLOCK(0, 128);
+  else if (dtype == 1 && dim == 64) RA_LAUNCH_BLOCK(1, 64);
+  else if (dtype == 1 && dim == 128) RA_LAUNCH_BLOCK(1, 128);
+#undef RA_LAUNCH_BLOCK
   else return hipErrorInvalidValue;
   return hipGetLastError();
 }
@@ -601,10 +636,16 @@ hipError_t launch_merge(const MergeArgs& a, int dtype, int dim, hipStream_t stre
   if (a.rows <= 0) return hipSuccess;
   const int rows_per_block = 256 / (dim / 8);
   const unsigned grid = (unsigned)((a.rows + rows_per_block - 1) / rows_per_block);
-  if (dtype == 0 && dim == 64) merge_kernel<0, 64><<<grid, 256, 0, stream>>>(a);
-  else if (dtype == 0 && dim == 128) merge_kernel<0, 128><<<grid, 256, 0, stream>>>(a);
-  else if (dtype == 1 && dim == 64) merge_kernel<1, 64><<<grid, 256, 0, stream>>>(a);
-  else if (dtype == 1 && dim == 128) merge_kernel<1, 128><<<grid, 256, 0, stream>>>(a);
+#define RA_LAUNCH_MERGE(DT_, D_)                                                 \
+  do {                                                                        \
+    if (a.half_partials) merge_kernel<DT_, D_, true><<<grid, 256, 0, stream>>>(a);  \
+    else merge_kernel<DT_, D_, false><<<grid, 256, 0, stream>>>(a);                \
+  } while (0)
+  if (dtype == 0 && dim == 64) RA_LAUNCH_MERGE(0, 64);
+  else if (dtype == 0 && dim == 128) RA_LAUNCH_MERGE(0, 128);
+  else if (dtype == 1 && dim == 64) RA_LAUNCH_MERGE(1, 64);
+  else if (dtype == 1 && dim == 128) RA_LAUNCH_MERGE(1, 128);
+#undef RA_LAUNCH_MERGE
   else return hipErrorInvalidValue;
   return hipGetLastError();
 }

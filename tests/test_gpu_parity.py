@@ -30,7 +30,8 @@ def to_dev(bits, dtype):
 
 
 def forward(w, q, k, v, **kw):
-    plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=w.graph, **kw)
+    plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=w.graph,
+                             half_partials=w.half_partials, **kw)
     try:
         out, lse = plan.forward(to_dev(q, w.dtype), to_dev(k, w.dtype), to_dev(v, w.dtype))
         torch.cuda.synchronize()
@@ -528,3 +529,45 @@ def test_maximum_ranks_long_sequence(oracle):
     out, lse = forward(w, q, k, v)
     assert torch.isfinite(out).all() and torch.isfinite(lse).all()
     check_rows(oracle, w, q, k, v, out, lse, sample_rows(w, 192))
+
+
+@pytest.mark.parametrize("w,layout", [
+    (Workload("hp_many_steps", 2, 4, 128, 16, 256, "fp16", 101, False), "contiguous"),
+    (Workload("hp_causal_bf16", 1, 4, 128, 4, 512, "bf16", 102, True), "contiguous"),
+    (Workload("hp_d64_zigzag", 2, 2, 64, 3, 384, "fp16", 103, True), "zigzag"),
+], ids=lambda x: x.name if isinstance(x, Workload) else x)
+def test_half_precision_partials(oracle, w, layout):
+    q, k, v = api.make_qkv_bits(w)
+    order = api.zigzag_order([w.chunk] * w.npes) if layout == "zigzag" else np.arange(w.seq)
+    inv = torch.from_numpy(np.argsort(order)).cuda()
+    qd, kd, vd = (to_dev(np.ascontiguousarray(x[:, :, order]), w.dtype) for x in (q, k, v))
+    full = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, layout=layout)
+    half = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, layout=layout, half_partials=True)
+    wb = half.lib.ringattn_workspace_bytes
+    assert wb(half.params) * (4 * w.dim + 4) == wb(full.params) * (2 * w.dim + 4)
+    o32, l32 = full.forward(qd, kd, vd)
+    o16, l16 = half.forward(qd, kd, vd)
+    torch.cuda.synchronize()
+    # same parity bar against the oracle, and close to the fp32-partial result: each merged part
+    # carries at most half an fp16 ulp of max |V|, plus one ulp of the output type
+    check_rows(oracle, w, q, k, v, o16[:, :, inv].contiguous(), l16[:, :, inv].contiguous(), np.arange(w.rows))
+    vmax = np.abs(bits_to_float64(v, w.dtype)).max()
+    ulp_out = 2.0**-10 if w.dtype == "fp16" else 2.0**-7
+    assert (o16.float() - o32.float()).abs().max().item() <= vmax * 2.0**-11 + ulp_out * vmax
+    assert torch.equal(l16, l32)                       # the partial LSEs stay fp32
+    # a step's fp16 partial is the fp32 partial rounded to nearest
+    for s in (0, w.npes - 1):
+        p32, pl32 = full.block_forward(s, qd, kd, vd)
+        p16, pl16 = half.block_forward(s, qd, kd, vd)
+        torch.cuda.synchronize()
+        assert p16.dtype == torch.float16 and torch.equal(p16, p32.half()) and torch.equal(pl16, pl32)
+    # merge of caller-held fp16 partials
+    parts = torch.zeros((w.npes,) + tuple(o16.shape), dtype=torch.float16, device="cuda")
+    lparts = torch.full((w.npes,) + tuple(l16.shape), float("-inf"), dtype=torch.float32, device="cuda")
+    for s in range(w.npes):
+        half.block_forward(s, qd, kd, vd, parts[s], lparts[s])
+    o_m, l_m = half.merge_ring(parts, lparts)
+    torch.cuda.synchronize()
+    assert torch.equal(o_m, o16) and torch.equal(l_m, l16)
+    full.close()
+    half.close()
