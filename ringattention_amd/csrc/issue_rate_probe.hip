@@ -54,29 +54,31 @@ __global__ __launch_bounds__(512) void probe(long long* ticks, float* sink, int 
         MFMA(acc0); MFMA(acc1); MFMA(acc0); MFMA(acc1);
       }
     } else if (MIX == kMfmaValu || MIX == kMfmaValuLds || MIX == kMfmaValuHalfLds) {
-      // per MFMA: 4 plain VALU ops and one exponential; per 4 MFMAs 4 KB (or 2 KB) of fragments,
-      // read one group of four MFMAs ahead of the wait
+      // The kernel's totals per 16 MFMAs: 48 plain VALU ops, 8 conversions, 8 max3, 16 exponentials
+      // (on rotating registers: no instruction waits for its neighbour), and 16 KB (or 8 KB) of
+      // fragments, each group of reads waited for four MFMAs after its issue.
 #pragma unroll
-      for (int r = 0; r < kRepeat; ++r) {
-        if (MIX == kMfmaValuLds) {
+      for (int g = 0; g < 4 * kRepeat; ++g) {
+        if ((g & 3) == 0 && MIX != kMfmaValu) {
           asm volatile("s_waitcnt lgkmcnt(0)" ::"v"(q0), "v"(q1), "v"(h0), "v"(h1), "v"(h2), "v"(h3) : "memory");
-          asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024" : "=v"(q0), "=v"(q1) : "v"(addr16));
-          asm volatile("ds_read_b64_tr_b16 %0, %4\n\tds_read_b64_tr_b16 %1, %4 offset:512\n\t"
-                       "ds_read_b64_tr_b16 %2, %4 offset:1024\n\tds_read_b64_tr_b16 %3, %4 offset:1536"
-                       : "=v"(h0), "=v"(h1), "=v"(h2), "=v"(h3) : "v"(addr8));
-        } else if (MIX == kMfmaValuHalfLds) {
-          asm volatile("s_waitcnt lgkmcnt(0)" ::"v"(q0), "v"(h0), "v"(h1) : "memory");
-          asm volatile("ds_read_b128 %0, %1" : "=v"(q0) : "v"(addr16));
-          asm volatile("ds_read_b64_tr_b16 %0, %2\n\tds_read_b64_tr_b16 %1, %2 offset:512" : "=v"(h0), "=v"(h1) : "v"(addr8));
+          if (MIX == kMfmaValuLds) {
+            asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024" : "=v"(q0), "=v"(q1) : "v"(addr16));
+            asm volatile("ds_read_b64_tr_b16 %0, %4\n\tds_read_b64_tr_b16 %1, %4 offset:512\n\t"
+                         "ds_read_b64_tr_b16 %2, %4 offset:1024\n\tds_read_b64_tr_b16 %3, %4 offset:1536"
+                         : "=v"(h0), "=v"(h1), "=v"(h2), "=v"(h3) : "v"(addr8));
+          } else {
+            asm volatile("ds_read_b128 %0, %1" : "=v"(q0) : "v"(addr16));
+            asm volatile("ds_read_b64_tr_b16 %0, %2\n\tds_read_b64_tr_b16 %1, %2 offset:512" : "=v"(h0), "=v"(h1) : "v"(addr8));
+          }
         }
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          if (g & 1) MFMA(acc1);
-          else MFMA(acc0);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) FMA(x[4 * g + i]);
-          EXP(x[4 * g]);
-        }
+        if (g & 1) MFMA(acc1);
+        else MFMA(acc0);
+        FMA(x[g & 15]);
+        FMA(x[(g + 1) & 15]);
+        FMA(x[(g + 2) & 15]);
+        if (g & 1) asm volatile("v_cvt_pk_bf16_f32 %0, %0, %0" : "+v"(x[(g + 4) & 15]));
+        else asm volatile("v_max3_f32 %0, %0, %0, %0" : "+v"(x[(g + 4) & 15]));
+        EXP(x[(g + 3) & 15]);
       }
     } else if (MIX == kExp) {
 #pragma unroll
@@ -133,7 +135,7 @@ int main(int argc, char** argv) {
   printf("two waves per SIMD, %d iterations; ticks = s_memtime counts per group of 4 MFMAs and wave\n", iters);
   printf("%-58s %8.1f ticks  MFMA utilisation 100.0 %%\n", "4 mfma_f32_32x32x16_bf16", mfma);
   const double v = run<kMfmaValu>(iters) / kRepeat;
-  printf("%-58s %8.1f ticks  MFMA utilisation %5.1f %%\n", "4 mfma + 16 v_fma_f32 + 4 v_exp_f32", v, 100 * mfma / v);
+  printf("%-58s %8.1f ticks  MFMA utilisation %5.1f %%\n", "4 mfma + 12 v_fma + 2 v_cvt_pk + 2 v_max3 + 4 v_exp", v, 100 * mfma / v);
   const double l = run<kMfmaValuLds>(iters) / kRepeat;
   printf("%-58s %8.1f ticks  MFMA utilisation %5.1f %%\n", "  + 2 ds_read_b128 + 4 ds_read_b64_tr_b16 (4 KB)", l, 100 * mfma / l);
   const double hl = run<kMfmaValuHalfLds>(iters) / kRepeat;
