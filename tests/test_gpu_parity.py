@@ -56,6 +56,11 @@ def check_rows(oracle, w, q, k, v, out, lse, rows, scale=None):
     assert np.isfinite(o_gpu).all() and np.isfinite(l_gpu).all()
     err_o = np.abs(o_gpu - o_ref).max()
     err_l = (np.abs(l_gpu - l_ref) / np.maximum(np.abs(l_ref), 1e-3)).max()
+    # also against the oracle rounded to the storage type (what a perfect kernel would store)
+    o_rounded = bits_to_float64(float32_to_bits(o_ref.astype(np.float32), w.dtype), w.dtype)
+    err_r = np.abs(o_gpu - o_rounded).max()
+    print(f"parity {w.name}: {len(rows)} rows, max|dO| = {err_o:.3e} vs fp64, {err_r:.3e} vs rounded fp64, "
+          f"max rel dLSE = {err_l:.3e}, max|O| = {np.abs(o_ref).max():.2f}")
     assert err_o <= O_TOL, f"{w.name}: max|dO| = {err_o:.3e}"
     assert err_l <= LSE_RTOL, f"{w.name}: max rel dLSE = {err_l:.3e}"
     return err_o, err_l
