@@ -78,7 +78,22 @@ def build_probe():
     return PROBE_PATH
 
 
+HARNESS_PATH = os.path.join(PKG_DIR, "reference_harness")
+
+
+def build_harness():
+    """Compile csrc/reference_harness.cpp (the reference's main() on the C ABI; host code linked to libringattn.so)."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    cmd = [hipcc, "-O2", "-std=c++17", "-I", os.path.join(REPO_DIR, "include"), os.path.join(CSRC, "reference_harness.cpp"),
+           "-o", HARNESS_PATH, "-L", PKG_DIR, "-l:libringattn.so", "-Wl,-rpath,$ORIGIN"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
+    return HARNESS_PATH
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
     print(build_probe())
+    print(build_harness())
     print(build_torch_shim(verbose=True))
