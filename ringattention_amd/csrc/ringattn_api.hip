@@ -249,6 +249,19 @@ void build_schedule(ringattn_plan* pl) {
   if (P < 4) n_groups = 1;
   else if (paired) n_groups = (P + 1) / 2 < kMaxGroups ? (P + 1) / 2 : kMaxGroups;
   else n_groups = P < 8 ? P / 2 : 4;
+  {
+    // Splitting only pays when every launch still fills the chip many times over: count the
+    // workgroups of the whole forward (128 query rows each) and keep at least 4096 per launch
+    // (8 rounds of 2 workgroups on each of 256 CUs).
+    std::vector<ringattn::WorkItem> all;
+    for (int r = 0; r < P; ++r)
+      for (int s = 0; s < P; ++s) append_items(all, d, P, causal, r, s);
+    int64_t wgs = 0;
+    for (const auto& w : all) wgs += (w.q_len + ringattn::kBlockM - 1) / ringattn::kBlockM;
+    wgs *= d.BH;
+    const int64_t fit = wgs / 4096;
+    if (fit < n_groups) n_groups = fit < 1 ? 1 : (int)fit;
+  }
   size_t pos = 0;
   for (int g = 0; g < n_groups; ++g) {
     // even split of the rank list; paired lists come in balanced pairs, keep pairs together
