@@ -31,6 +31,22 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
+@pytest.fixture(scope="session", autouse=True)
+def built_artifacts():
+    """The tests load what is built; only where a build product is missing altogether (a fresh
+    checkout) is it compiled here, once per session."""
+    from ringattention_amd import _build
+    if not os.path.exists(_build.LIB_PATH):
+        _build.build_library()
+    if not os.path.exists(_build.TORCH_LIB_PATH):
+        _build.build_torch_shim()
+    if not os.path.exists(_build.HARNESS_PATH):
+        _build.build_harness()
+    from oracle import build as oracle_build
+    if not os.path.exists(oracle_build.LIB_PATH):
+        oracle_build.build_oracle()
+
+
 @pytest.fixture(scope="session")
 def oracle():
     from oracle import oracle as o
