@@ -160,6 +160,32 @@ int ringattn_merge_ring(ringattn_plan* plan, const void* o_parts, const float* l
                         void* out, float* lse, void* stream);
 
 /*
+ * One ring step of ONE rank on rank-local buffers -- what a process of the reference does in
+ * one iteration of its step loop (csrc/ring_attention.cu:456-620) once the K/V chunk of rank
+ * (rank + step) mod npes has arrived (:611-619):
+ *   q        : [batch, heads, h_seqlen[rank], dim]       the rank's own queries
+ *   k_chunk,
+ *   v_chunk  : [batch, kv_heads, h_seqlen[j], dim]       the visited chunk, j = (rank + step) mod npes
+ *   o_part   : [batch, heads, h_seqlen[rank], dim] fp32 (fp16 with RINGATTN_FLAG_HALF_PARTIALS)
+ *   lse_part : [batch, heads, h_seqlen[rank]] fp32
+ * Rows that see no key of the visited chunk are left untouched (nothing at all is launched if
+ * that holds for the whole rank).  The results are bit-identical to the rows ringattn_block_fwd
+ * writes for this rank in this step.  This is the call a one-process-per-GPU ring makes between
+ * its K/V exchanges; the exchange itself is the caller's.
+ */
+int ringattn_rank_step_fwd(ringattn_plan* plan, int rank, int step, const void* q, const void* k_chunk,
+                           const void* v_chunk, void* o_part, float* lse_part, void* stream);
+
+/*
+ * The merge of one rank's per-step partials: o_parts [npes, batch*heads*h_seqlen[rank], dim] and
+ * lse_parts [npes, batch*heads*h_seqlen[rank]], slot s as written by ringattn_rank_step_fwd for
+ * step s (slots of steps that left the rows untouched are not read); out / lse hold the rank's
+ * rows only.  Bit-identical to the rows ringattn_fwd produces for this rank.
+ */
+int ringattn_rank_merge(ringattn_plan* plan, int rank, const void* o_parts, const float* lse_parts, void* out,
+                        float* lse, void* stream);
+
+/*
  * The schedule of a plan, for inspection (host data, no GPU work; the reference has no
  * counterpart: its schedule is the loop `for step in 0..npes-1: kv_pe = (mype + step) % npes`
  * of csrc/ring_attention.cu:456-470,615).  A work item is one block-attention job: the

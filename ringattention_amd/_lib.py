@@ -48,6 +48,8 @@ SYMBOLS = {
     "ringattn_merge": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
                                       ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
     "ringattn_merge_ring": (ctypes.c_int, [ctypes.c_void_p] * 6),
+    "ringattn_rank_step_fwd": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int] + [ctypes.c_void_p] * 6),
+    "ringattn_rank_merge": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 5),
     "ringattn_plan_work_items": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(RingattnWorkItem),
                                                 ctypes.c_int, c_int_p]),
     "ringattn_plan_launch_times": (ctypes.c_int, [ctypes.c_void_p, c_float_p, ctypes.c_int, c_int_p]),

@@ -123,6 +123,33 @@ class RingAttention:
                                           _ptr(lse_part), _stream_ptr(stream)), "ringattn_block_fwd")
         return o_part, lse_part
 
+    def rank_step_forward(self, rank, step, q, k_chunk, v_chunk, o_part=None, lse_part=None, stream=None):
+        """One ring step of one rank on rank-local tensors (q: the rank's rows; k_chunk, v_chunk: the
+        chunk of rank (rank + step) % npes).  Returns the rank-local partial (O, LSE)."""
+        rows = self.seqlen[rank]
+        for t, nm in ((q, "q"), (k_chunk, "k_chunk"), (v_chunk, "v_chunk")):
+            _check_tensor(t, nm, self.torch_dtype)
+        if o_part is None:
+            o_part = torch.zeros((self.batch, self.heads, rows, self.dim), dtype=self.part_dtype, device=q.device)
+        if lse_part is None:
+            lse_part = torch.full((self.batch, self.heads, rows), float("-inf"), dtype=torch.float32, device=q.device)
+        check(self.lib.ringattn_rank_step_fwd(self.handle, int(rank), int(step), _ptr(q), _ptr(k_chunk), _ptr(v_chunk),
+                                              _ptr(o_part), _ptr(lse_part), _stream_ptr(stream)), "ringattn_rank_step_fwd")
+        return o_part, lse_part
+
+    def rank_merge(self, rank, o_parts, lse_parts, out=None, lse=None, stream=None):
+        """Merge of one rank's per-step partials [npes, B, H, rows, d] / [npes, B, H, rows]."""
+        rows = self.seqlen[rank]
+        _check_tensor(o_parts, "o_parts", self.part_dtype)
+        _check_tensor(lse_parts, "lse_parts", torch.float32)
+        if out is None:
+            out = torch.empty((self.batch, self.heads, rows, self.dim), dtype=self.torch_dtype, device=o_parts.device)
+        if lse is None:
+            lse = torch.empty((self.batch, self.heads, rows), dtype=torch.float32, device=o_parts.device)
+        check(self.lib.ringattn_rank_merge(self.handle, int(rank), _ptr(o_parts), _ptr(lse_parts), _ptr(out), _ptr(lse),
+                                           _stream_ptr(stream)), "ringattn_rank_merge")
+        return out, lse
+
     def launch_times(self):
         """Milliseconds of each block-attention launch of the last forward (plan made with timing=True)."""
         ms = (ctypes.c_float * 8)()

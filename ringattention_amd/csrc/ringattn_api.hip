@@ -170,6 +170,8 @@ struct ringattn_plan {
   std::vector<MergeRegion> regions;  // group by group, then (from all_regions on) rank by rank
   int all_regions = 0;
   std::vector<int> step_begin;       // [npes + 1] slices of h_items, one per ring step
+  std::vector<int> local_begin;      // [npes * npes + 1] slices of h_items: the items of (rank, step) in
+                                     // rank-local rows (queries from 0, keys from 0 of the visited chunk)
   int q_tiles_max = 0;
   ringattn::WorkItem* d_items = nullptr;
   hipStream_t merge_stream = nullptr;
@@ -290,6 +292,20 @@ void build_schedule(ringattn_plan* pl) {
     for (int r = 0; r < P; ++r) append_items(pl->h_items, d, P, causal, r, s);
   }
   pl->step_begin.push_back((int)pl->h_items.size());
+  // rank-local lists for ringattn_rank_step_fwd: one (rank, step) at a time, rows counted from the
+  // start of the rank's own chunk and of the visited chunk, one partial slot
+  for (int r = 0; r < P; ++r)
+    for (int s = 0; s < P; ++s) {
+      pl->local_begin.push_back((int)pl->h_items.size());
+      const size_t first = pl->h_items.size();
+      append_items(pl->h_items, d, P, causal, r, s);
+      for (size_t i = first; i < pl->h_items.size(); ++i) {
+        pl->h_items[i].q_start -= d.start[r];
+        pl->h_items[i].kv_start -= d.start[(r + s) % P];
+        pl->h_items[i].slot = 0;
+      }
+    }
+  pl->local_begin.push_back((int)pl->h_items.size());
   int longest = 0;
   for (const auto& w : pl->h_items) longest = w.q_len > longest ? w.q_len : longest;
   pl->q_tiles_max = (longest + ringattn::kBlockM - 1) / ringattn::kBlockM;
@@ -536,6 +552,66 @@ int ringattn_merge_ring(ringattn_plan* plan, const void* o_parts, const float* l
   for (size_t i = (size_t)plan->all_regions; i < plan->regions.size(); ++i) {
     int rc = launch_region_merge(plan, o_parts, lse_parts, out, lse, (hipStream_t)stream, plan->regions[i]);
     if (rc != RINGATTN_OK) return rc;
+  }
+  return RINGATTN_OK;
+}
+
+int ringattn_rank_step_fwd(ringattn_plan* plan, int rank, int step, const void* q, const void* k_chunk,
+                           const void* v_chunk, void* o_part, float* lse_part, void* stream) {
+  if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
+  if (!q || !k_chunk || !v_chunk || !o_part || !lse_part) return RINGATTN_ERR_NULL;
+  const int P = plan->p.npes;
+  if (rank < 0 || rank >= P || step < 0 || step >= P) return RINGATTN_ERR_RANK;
+  if (!aligned16(q) || !aligned16(k_chunk) || !aligned16(v_chunk) || !aligned16(o_part) || ((uintptr_t)lse_part & 3u)) return RINGATTN_ERR_ALIGN;
+  int rc = ensure_streams(plan);
+  if (rc != RINGATTN_OK) return rc;
+  const int begin = plan->local_begin[rank * P + step], count = plan->local_begin[rank * P + step + 1] - begin;
+  if (count == 0) return RINGATTN_OK;  // nothing of the visited chunk is visible to this rank
+  const Derived& d = plan->d;
+  const int j = (rank + step) % P;
+  const int64_t q_rows = d.start[rank + 1] - d.start[rank], kv_rows = d.start[j + 1] - d.start[j];
+  ringattn::BlockStepArgs a;
+  fill_geometry(a, plan->p, d);
+  a.q = q;
+  a.k = k_chunk;
+  a.v = v_chunk;
+  a.o_part = o_part;
+  a.lse_part = lse_part;
+  a.items = plan->d_items + begin;
+  a.n_items = count;
+  a.bh_stride = q_rows * plan->p.dim;      // every tensor holds one rank's rows only
+  a.kv_bh_stride = kv_rows * plan->p.dim;
+  a.S = (int)q_rows;
+  a.part_stride_rows = d.BH * q_rows;
+  a.q_tiles_max = (int)((q_rows + ringattn::kBlockM - 1) / ringattn::kBlockM);
+  RA_HIP(ringattn::launch_block_step(a, plan->p.dtype, plan->p.dim, (hipStream_t)stream));
+  return RINGATTN_OK;
+}
+
+int ringattn_rank_merge(ringattn_plan* plan, int rank, const void* o_parts, const float* lse_parts, void* out,
+                        float* lse, void* stream) {
+  if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
+  if (!o_parts || !lse_parts || !out || !lse) return RINGATTN_ERR_NULL;
+  if (rank < 0 || rank >= plan->p.npes) return RINGATTN_ERR_RANK;
+  if (!aligned16(o_parts) || !aligned16(out) || ((uintptr_t)lse_parts & 3u) || ((uintptr_t)lse & 3u)) return RINGATTN_ERR_ALIGN;
+  const Derived& d = plan->d;
+  const int r0 = d.start[rank], r1 = d.start[rank + 1];
+  for (size_t i = (size_t)plan->all_regions; i < plan->regions.size(); ++i) {
+    const MergeRegion& reg = plan->regions[i];
+    if (reg.start < r0 || reg.start >= r1) continue;
+    ringattn::MergeArgs m;
+    m.o_parts = o_parts;
+    m.lse_parts = lse_parts;
+    m.out = out;
+    m.lse = lse;
+    m.sel_start = reg.start - r0;
+    m.sel_len = reg.len;
+    m.rows = d.BH * reg.len;
+    m.S = r1 - r0;
+    m.part_stride_rows = d.BH * (int64_t)(r1 - r0);
+    m.active = reg.active;
+    m.half_partials = half_partials(plan->p) ? 1 : 0;
+    RA_HIP(ringattn::launch_merge(m, plan->p.dtype, plan->p.dim, (hipStream_t)stream));
   }
   return RINGATTN_OK;
 }

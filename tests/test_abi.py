@@ -100,8 +100,16 @@ def test_plan_lifetime_with_caller_workspace(ralib):
     assert ralib.ringattn_block_fwd(h, 2, x, x, x, x, x, None) == E_RANK
     assert ralib.ringattn_block_fwd(h, -1, x, x, x, x, x, None) == E_RANK
     assert ralib.ringattn_block_fwd(h, 0, x, x, None, x, x, None) == E_NULL
+    # the rank-local entry points
+    assert ralib.ringattn_rank_step_fwd(h, 2, 0, x, x, x, x, x, None) == E_RANK
+    assert ralib.ringattn_rank_step_fwd(h, 0, -1, x, x, x, x, x, None) == E_RANK
+    assert ralib.ringattn_rank_step_fwd(h, 0, 0, x, None, x, x, x, None) == E_NULL
+    assert ralib.ringattn_rank_step_fwd(h, 0, 0, x, x, x, ctypes.c_void_p(base + 8), x, None) == E_ALIGN
+    assert ralib.ringattn_rank_merge(h, 5, x, x, x, x, None) == E_RANK
+    assert ralib.ringattn_rank_merge(h, 0, x, x, None, x, None) == E_NULL
     assert ralib.ringattn_plan_destroy(h) == OK
     assert ralib.ringattn_plan_destroy(h) == E_PLAN          # double destroy
+    assert ralib.ringattn_rank_step_fwd(h, 0, 0, x, x, x, x, x, None) == E_PLAN
     assert ralib.ringattn_fwd(h, x, x, x, x, x, None) == E_PLAN  # use after destroy
     assert ralib.ringattn_plan_destroy(None) == E_PLAN
 

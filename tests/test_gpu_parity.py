@@ -576,3 +576,39 @@ def test_half_precision_partials(oracle, w, layout):
     assert torch.equal(o_m, o16) and torch.equal(l_m, l16)
     full.close()
     half.close()
+
+
+@pytest.mark.parametrize("seqlen,causal,layout,d,dtype,hkv,half", [
+    ((256, 256, 256, 256), True, "contiguous", 128, "bf16", 0, False),
+    ((256, 256, 256, 256), False, "contiguous", 64, "fp16", 0, False),
+    ((512, 256, 768), True, "zigzag", 128, "bf16", 2, False),
+    ((100, 334, 2, 78), True, "zigzag", 128, "fp16", 0, True),
+    ((100, 333, 1, 77), True, "contiguous", 64, "bf16", 0, False),
+])
+def test_rank_local_ring_equals_the_all_rank_forward(seqlen, causal, layout, d, dtype, hkv, half):
+    # A ring of one process per GPU, replayed rank by rank on this GPU: every rank holds only its
+    # own Q rows and, at step s, the K/V chunk of rank (r + s) mod P in a buffer of its own (what
+    # the exchange would have delivered).  Same work items, so the same bits as ringattn_fwd.
+    P, S, B, H = len(seqlen), sum(seqlen), 2, 4
+    w = Workload("rank_local", B, H, d, 1, S, dtype, 111, causal)
+    q, _, _ = api.make_qkv_bits(w)
+    _, k, v = api.make_qkv_bits(Workload("rank_local_kv", B, hkv or H, d, 1, S, dtype, 112, causal))
+    qd, kd, vd = (to_dev(x, dtype) for x in (q, k, v))
+    plan = api.RingAttention(P, list(seqlen), d, B, H, dtype, causal, kv_heads=hkv, layout=layout, half_partials=half)
+    out, lse = plan.forward(qd, kd, vd)
+    torch.cuda.synchronize()
+    start = np.concatenate([[0], np.cumsum(seqlen)])
+    for r in range(P):
+        rows = slice(start[r], start[r + 1])
+        q_r = qd[:, :, rows].contiguous()
+        o_parts = torch.zeros((P, B, H, seqlen[r], d), dtype=plan.part_dtype, device="cuda")
+        l_parts = torch.full((P, B, H, seqlen[r]), float("-inf"), dtype=torch.float32, device="cuda")
+        for s in range(P):
+            j = (r + s) % P
+            k_j = kd[:, :, start[j]:start[j + 1]].contiguous()      # the chunk the ring delivered
+            v_j = vd[:, :, start[j]:start[j + 1]].contiguous()
+            plan.rank_step_forward(r, s, q_r, k_j, v_j, o_parts[s], l_parts[s])
+        o_r, l_r = plan.rank_merge(r, o_parts, l_parts)
+        torch.cuda.synchronize()
+        assert torch.equal(o_r, out[:, :, rows]) and torch.equal(l_r, lse[:, :, rows]), f"rank {r}"
+    plan.close()
