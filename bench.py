@@ -49,6 +49,8 @@ def main():
     ap.add_argument("--workload", default="cfg4")
     ap.add_argument("--layout", default="contiguous", choices=["contiguous", "zigzag"],
                     help="placement of the sequence on the ranks (zigzag: load-balanced causal ring)")
+    ap.add_argument("--rank-local", action="store_true",
+                    help="also time the ring rank by rank on rank-local buffers (one launch per rank and step)")
     ap.add_argument("--per-step", action="store_true", help="also time one block-attention launch per ring step")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the cpu_baseline sample (0 = skip)")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
@@ -159,6 +161,46 @@ def main():
         per_step = {"ms": [round(float(x), 4) for x in step_ms],
                     "tflops": [round(f / (t * 1e-3) / 1e12, 1) for f, t in zip(step_flops, step_ms)]}
     del o_parts, l_parts
+
+    # ---- optional: the ring as one process per GPU would run it, replayed rank by rank on this
+    # GPU with rank-local buffers (ringattn_rank_step_fwd / ringattn_rank_merge): every launch is one
+    # (rank, step), i.e. the kernel on one GPU's share at its real shape.  In a real ring the ranks
+    # move in lockstep (one K/V exchange per step), so a step costs what its slowest rank costs.
+    ring = None
+    if args.rank_local:
+        P, c = w.npes, w.chunk
+        kvh = w.heads
+        t_step = np.zeros((P, P))
+        t_merge = np.zeros(P)
+        for r in range(P):
+            q_r = qd[:, :, r * c:(r + 1) * c].contiguous()
+            op = torch.zeros((P, w.batch, w.heads, c, w.dim), dtype=eager.part_dtype, device="cuda")
+            lp = torch.full((P, w.batch, w.heads, c), float("-inf"), dtype=torch.float32, device="cuda")
+            o_r = torch.empty((w.batch, w.heads, c, w.dim), dtype=qd.dtype, device="cuda")
+            l_r = torch.empty((w.batch, w.heads, c), dtype=torch.float32, device="cuda")
+            chunks = [(kd[:, :, j * c:(j + 1) * c].contiguous(), vd[:, :, j * c:(j + 1) * c].contiguous()) for j in range(P)]
+            e = [[torch.cuda.Event(enable_timing=True) for _ in range(P + 2)] for _ in range(reps)]
+            for rep in range(-1, reps):
+                for st in range(P):
+                    if rep >= 0:
+                        e[rep][st].record(stream)
+                    kj, vj = chunks[(r + st) % P]
+                    eager.rank_step_forward(r, st, q_r, kj, vj, op[st], lp[st], stream)
+                if rep >= 0:
+                    e[rep][P].record(stream)
+                eager.rank_merge(r, op, lp, o_r, l_r, stream)
+                if rep >= 0:
+                    e[rep][P + 1].record(stream)
+            torch.cuda.synchronize()
+            for st in range(P):
+                t_step[r, st] = np.mean([e[k][st].elapsed_time(e[k][st + 1]) for k in range(reps)])
+            t_merge[r] = np.mean([e[k][P].elapsed_time(e[k][P + 1]) for k in range(reps)])
+            del q_r, op, lp, o_r, l_r, chunks
+        lockstep = float(t_step.max(axis=0).sum() + t_merge.max())
+        ring = {"per_rank_ms": [round(float(x), 4) for x in (t_step.sum(axis=1) + t_merge)],
+                "per_step_slowest_rank_ms": [round(float(x), 4) for x in t_step.max(axis=0)],
+                "lockstep_ms": round(lockstep, 4),
+                "per_gpu_tflops_in_lockstep": round(w.flops / P / (lockstep * 1e-3) / 1e12, 1)}
     eager.close()
     plan.close()
 
@@ -191,7 +233,7 @@ def main():
         "config": {"workload": describe(w), "algorithmic_flop": w.flops, "graph": bool(w.graph), "layout": args.layout,
                    "partials": "fp16" if w.half_partials else "fp32"},
         "pct_mfma_peak": round(100.0 * tflops / peak, 2),
-        "roofline": roofline, "merge": merge, "per_ring_step": per_step, "cpu_baseline": cpu,
+        "roofline": roofline, "merge": merge, "per_ring_step": per_step, "rank_local_ring": ring, "cpu_baseline": cpu,
     }))
 
 
