@@ -224,3 +224,17 @@ def test_zigzag_order_small_case():
     o = zigzag_order([256, 768, 512])
     assert sorted(o.tolist()) == list(range(1536))
     assert o[:128].tolist() == list(range(128)) and o[128] == 1536 - 128   # rank 0: first low half, last high half
+
+
+def test_header_is_plain_c(tmp_path):
+    # the boundary is a C ABI: the header must compile as C99 (no C++, no HIP, no torch types)
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "ringattn.h"\nint main(void) { ringattn_params p; (void)p; return ringattn_strerror(0) == 0; }\n')
+    res = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+                          "-c", str(src), "-o", str(tmp_path / "use_header.o")], capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
