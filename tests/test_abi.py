@@ -238,3 +238,34 @@ def test_header_is_plain_c(tmp_path):
     res = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
                           "-c", str(src), "-o", str(tmp_path / "use_header.o")], capture_output=True, text=True)
     assert res.returncode == 0, res.stderr
+
+
+def test_plans_from_many_threads(ralib):
+    # the live-plan registry is shared: creating, inspecting and destroying plans from several
+    # threads at once must neither crash nor confuse handles
+    import threading
+    errors = []
+
+    def worker(seed):
+        try:
+            rng = np.random.default_rng(seed)
+            for _ in range(200):
+                P = int(rng.integers(1, 9))
+                lens = tuple(int(2 * rng.integers(1, 300)) for _ in range(P))
+                causal = int(rng.integers(0, 2))
+                h = _plan_on_host(ralib, params(npes=P, seqlen=lens, causal=causal, layout=int(rng.integers(0, 2))))
+                items = _work_items(ralib, h, -1)
+                want = sum(1 for r in range(P) for s in range(P) if not causal or (r + s) % P <= r) if not causal else None
+                if not causal:
+                    assert len(items) == P * P == want
+                assert ralib.ringattn_plan_destroy(h) == OK
+                assert ralib.ringattn_plan_destroy(h) == E_PLAN
+        except Exception as e:   # noqa: BLE001 - reported below
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
