@@ -421,14 +421,15 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
     }
   };
 
-  __builtin_amdgcn_s_waitcnt(0);  // retire the Q loads with a wait the compiler can see
+  // the first tiles go out next to the Q loads: one memory latency for all of them
   issue_k(0, kChecked);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
   if (n_tiles > 1) issue_k(1, kChecked);
   if (n_tiles > 2) issue_k(2, kChecked);
   issue_v(0, kChecked);
   if (n_tiles > 1) issue_v(1, kChecked);
+  __builtin_amdgcn_s_waitcnt(0);  // retire the Q loads with a wait the compiler can see (and the tiles)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
   {
     float cand[QB];
     qk(s_even, 0);
