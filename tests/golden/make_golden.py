@@ -21,7 +21,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
-from np_reference import float32_to_bits, np_fill_normal, np_make_qkv, torch_attention  # noqa: E402
+from np_reference import np_fill_normal, np_make_qkv, torch_attention  # noqa: E402
 from ringattention_amd.configs import WORKLOADS, Workload  # noqa: E402
 
 HERE = os.path.dirname(os.path.abspath(__file__))

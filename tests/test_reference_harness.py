@@ -7,7 +7,6 @@ import subprocess
 import numpy as np
 import pytest
 
-from np_reference import bits_to_float64
 from ringattention_amd import api
 from ringattention_amd._build import HARNESS_PATH
 

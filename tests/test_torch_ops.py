@@ -1,5 +1,4 @@
 """The torch front end (dispatcher op ringattn::fwd over the C ABI)."""
-import numpy as np
 import pytest
 import torch
 
