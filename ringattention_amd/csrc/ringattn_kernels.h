@@ -13,7 +13,7 @@ constexpr int kMaxParts = 64; // partial slots a merge can combine
 // against the keys/values [kv_start, kv_start + kv_len) of the matching KV head -- the body
 // of one ring step of one rank (csrc/ring_attention.cu:456-470,531-610: rank r at step s
 // works on the KV chunk of rank (r + s) mod P).  Row numbers are local to a head's [S, D]
-// slab; all four are multiples of kBlockM.  The normalised partial O and the partial LSE
+// slab and need not be multiples of any tile size.  The normalised partial O and the partial LSE
 // of the item go to partial slot `slot`, at the rows of its queries.
 struct WorkItem {
   int q_start, q_len;

@@ -49,9 +49,11 @@ typedef short s16x8 __attribute__((ext_vector_type(8)));
 // kernel waits for it explicitly (s_waitcnt vmcnt(0)) before the tile barrier.
 // No "memory" clobber: a transfer only ever targets a ring slot that no LDS read between
 // the surrounding barriers touches, so the compiler may move LDS reads across it.
-// Nothing else in these kernels uses M0.
+// M0 is declared clobbered, and the s_nop is the wait state the hardware needs between a
+// scalar write of M0 and the LDS-DMA instruction that reads it (the assembler inserts none
+// inside inline asm).
 static __device__ __forceinline__ void load_lds_16(const void* base, int voff, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base));
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "m0");
 }
 static __device__ __forceinline__ unsigned lds_offset(const void* p) {
   return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
