@@ -235,6 +235,27 @@ int ringattn_ring_attention(const void* q, const void* k, const void* v, void* o
                             int dtype, int causal, float softmax_scale);
 
 /*
+ * ringattn_ring_attention for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference (whose entry allocates on every call, csrc/ring_attention.cu:383-394).  Same
+ * arguments and results as ringattn_ring_attention, plus the stream; it calls no hipMalloc,
+ * hipFree, memcpy or other allocating routine and does not synchronise: the work (a
+ * table-writing kernel, the block kernel, the merge) is queued on `stream`.  The per-step
+ * partials live in a static device array of ringattn_noalloc_scratch_bytes() bytes (32 MiB,
+ * held by every GPU the library runs on until the process ends); a call that needs more --
+ * visible_steps * (seqlen[mype] * (dim + 1) * 4 + 32) + seqlen[mype] * 4 bytes, visible_steps
+ * being npes, or mype + 1 with the causal mask -- returns RINGATTN_ERR_WORKSPACE.  All calls on
+ * one GPU share that array: calls that overlap on one GPU (two streams, two threads) race;
+ * nothing in it needs clearing between calls.
+ */
+int ringattn_ring_attention_noalloc(const void* q, const void* k, const void* v, void* out, float* lse,
+                                    int npes, int mype, const int* seqlen, int dim, int max_seq,
+                                    int dtype, int causal, float softmax_scale, void* stream);
+
+/* Size in bytes of the static device scratch behind ringattn_ring_attention_noalloc. */
+size_t ringattn_noalloc_scratch_bytes(void);
+
+/*
  * Seeded input generator -- the counterpart of fillWithNum / initQKV
  * (csrc/ring_attention.cu:731-748), which fill a host buffer and copy it to the
  * device.  Writes n values of N(0, sigma^2), rounded to nearest-even into `dtype`,

@@ -58,6 +58,10 @@ SYMBOLS = {
     "ringattn_ring_attention": (ctypes.c_int, [ctypes.c_void_p] * 5 + [ctypes.c_int, ctypes.c_int, c_int_p,
                                                                        ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                                        ctypes.c_int, ctypes.c_float]),
+    "ringattn_ring_attention_noalloc": (ctypes.c_int, [ctypes.c_void_p] * 5 + [ctypes.c_int, ctypes.c_int, c_int_p,
+                                                                               ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                                               ctypes.c_int, ctypes.c_float, ctypes.c_void_p]),
+    "ringattn_noalloc_scratch_bytes": (ctypes.c_size_t, []),
     "ringattn_fill_normal": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_uint64,
                                             ctypes.c_int64, ctypes.c_double]),
     "ringattn_fill_reference_pattern": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int]),

@@ -238,6 +238,22 @@ def ring_attention(q, k, v, out, npes, mype, seqlen, dim, max_seq, lse=None, cau
     return out
 
 
+def ring_attention_noalloc(q, k, v, out, npes, mype, seqlen, dim, max_seq, lse=None, causal=False, softmax_scale=0.0,
+                           stream=None):
+    """ring_attention() through the entry point that allocates nothing (static device scratch);
+    asynchronous on `stream`.  Raises RingattnError (workspace) if the rank's partials do not fit."""
+    lib = _lib.load()
+    for t, nm in ((q, "q"), (k, "k"), (v, "v"), (out, "out")):
+        _check_tensor(t, nm, q.dtype)
+    arr = (ctypes.c_int * len(seqlen))(*[int(x) for x in seqlen])
+    check(lib.ringattn_ring_attention_noalloc(_ptr(q), _ptr(k), _ptr(v), _ptr(out),
+                                              _ptr(lse) if lse is not None else None, int(npes), int(mype), arr,
+                                              int(dim), int(max_seq), DTYPE_CODE[q.dtype], int(bool(causal)),
+                                              float(softmax_scale), _stream_ptr(stream)),
+          "ringattn_ring_attention_noalloc")
+    return out
+
+
 # ---- seeded inputs (counterpart of fillWithNum / initQKV, csrc/ring_attention.cu:731-748) ----
 
 def fill_normal(n, dtype, seed, offset=0, sigma=1.0):

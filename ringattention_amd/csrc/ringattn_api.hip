@@ -413,6 +413,107 @@ inline bool plan_ok(const ringattn_plan* pl) {
   return g_plans.count(pl) != 0;
 }
 
+
+// ---- the reference-shaped call for one rank (ringattn_ring_attention and its variant that
+// allocates nothing) ------------------------------------------------------------------------
+// Device scratch of one call: the rank's per-step partial O [n_parts, c, dim] fp32, partial LSE
+// [n_parts, c], a spare LSE row [c] for callers that pass no lse, and the item table.
+struct RankCall {
+  ringattn_params p;
+  Derived d;
+  ringattn::ItemPack pack;  // the visible ring steps of the rank in ring order, one compact slot each
+  int n_parts = 0;
+  int c = 0;                // rows of this rank
+  size_t lse_floats = 0;    // floats of the two LSE areas, padded so the item table stays 32-byte aligned
+  size_t scratch_bytes = 0;
+};
+
+int prepare_rank_call(RankCall* rc, const void* q, const void* k, const void* v, void* out, int npes, int mype,
+                      const int* seqlen, int dim, int max_seq, int dtype, int causal, float softmax_scale) {
+  ringattn_params& p = rc->p;
+  std::memset(&p, 0, sizeof(p));
+  p.npes = npes;
+  p.h_seqlen = seqlen;
+  p.dim = dim;
+  p.softmax_scale = softmax_scale;
+  p.batch = 1;
+  p.heads = 1;
+  p.dtype = dtype;
+  p.causal = causal;
+  int err = validate(&p, &rc->d);
+  if (err != RINGATTN_OK) return err;
+  const Derived& d = rc->d;
+  if (mype < 0 || mype >= npes) return RINGATTN_ERR_RANK;
+  if (max_seq < d.max_len) return RINGATTN_ERR_SEQLEN;
+  if (!q || !k || !v || !out) return RINGATTN_ERR_NULL;
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return RINGATTN_ERR_ALIGN;
+  // the query rows are local to the caller's rank-sized q and out buffers
+  rc->c = d.start[mype + 1] - d.start[mype];
+  rc->n_parts = 0;
+  for (int s = 0; s < npes; ++s) {
+    const int j = (mype + s) % npes;
+    if (causal && j > mype) continue;
+    rc->pack.items[rc->n_parts] =
+        make_item(0, rc->c, d.start[j], d.start[j + 1] - d.start[j], (causal && j == mype) ? 0 : -1, rc->n_parts);
+    ++rc->n_parts;
+  }
+  rc->lse_floats = ((size_t)(rc->n_parts + 1) * rc->c + 7) & ~(size_t)7;
+  rc->scratch_bytes = ((size_t)rc->n_parts * rc->c * dim + rc->lse_floats) * sizeof(float) +
+                      (size_t)rc->n_parts * sizeof(ringattn::WorkItem);
+  return RINGATTN_OK;
+}
+
+// Item table (written by a kernel from its arguments), block kernel, merge: three launches on
+// `stream`, nothing is allocated or copied from the host.  `scratch`: rc.scratch_bytes of device memory.
+int run_rank_call(const RankCall& rc, void* scratch, const void* q, const void* k, const void* v, void* out,
+                  float* lse, hipStream_t stream) {
+  const int dim = rc.p.dim, c = rc.c, n_parts = rc.n_parts;
+  float* o_parts = (float*)scratch;
+  float* lse_parts = o_parts + (size_t)n_parts * c * dim;
+  float* lse_tmp = lse_parts + (size_t)n_parts * c;
+  ringattn::WorkItem* d_items = (ringattn::WorkItem*)(lse_parts + rc.lse_floats);
+  RA_HIP(ringattn::launch_write_items(rc.pack, n_parts, d_items, stream));
+  ringattn::BlockStepArgs a;
+  fill_geometry(a, rc.p, rc.d);
+  a.q = q;
+  a.k = k;
+  a.v = v;
+  a.o_part = o_parts;
+  a.lse_part = lse_parts;
+  a.items = d_items;
+  a.n_items = n_parts;
+  a.q_tiles_max = (c + ringattn::kBlockM - 1) / ringattn::kBlockM;
+  a.bh_stride = (int64_t)c * dim;
+  a.part_stride_rows = c;
+  a.S = c;
+  RA_HIP(ringattn::launch_block_step(a, rc.p.dtype, dim, stream));
+  return ringattn_merge(o_parts, lse_parts, n_parts, (int64_t)c, dim, rc.p.dtype, out, lse ? lse : lse_tmp, stream);
+}
+
+// Static device scratch of ringattn_ring_attention_noalloc.  In host code the array's name is
+// only a handle for hipGetSymbolAddress; the device address is looked up once per device
+// (each GPU holds its own copy of the array) and kept.
+constexpr size_t kScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int device_scratch(void** base) {
+  int dev = -1;
+  RA_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return RINGATTN_ERR_SHAPE;
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    RA_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return RINGATTN_ERR_HIP;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *base = g_scratch_ptr[dev];
+  return RINGATTN_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -684,67 +785,32 @@ int ringattn_merge(const float* o_parts, const float* lse_parts, int n_parts, in
 int ringattn_ring_attention(const void* q, const void* k, const void* v, void* out, float* lse,
                             int npes, int mype, const int* seqlen, int dim, int max_seq,
                             int dtype, int causal, float softmax_scale) {
-  ringattn_params p;
-  std::memset(&p, 0, sizeof(p));
-  p.npes = npes;
-  p.h_seqlen = seqlen;
-  p.dim = dim;
-  p.softmax_scale = softmax_scale;
-  p.batch = 1;
-  p.heads = 1;
-  p.dtype = dtype;
-  p.causal = causal;
-  Derived d;
-  int rc = validate(&p, &d);
+  RankCall rc_;
+  int rc = prepare_rank_call(&rc_, q, k, v, out, npes, mype, seqlen, dim, max_seq, dtype, causal, softmax_scale);
   if (rc != RINGATTN_OK) return rc;
-  if (mype < 0 || mype >= npes) return RINGATTN_ERR_RANK;
-  if (max_seq < d.max_len) return RINGATTN_ERR_SEQLEN;
-  if (!q || !k || !v || !out) return RINGATTN_ERR_NULL;
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return RINGATTN_ERR_ALIGN;
-
-  // the visible ring steps of rank mype in ring order, one compact partial slot each; the
-  // query rows are local to the caller's rank-sized q and out buffers
-  const int c = d.start[mype + 1] - d.start[mype];  // rows of this rank
-  std::vector<ringattn::WorkItem> items;
-  for (int s = 0; s < npes; ++s) {
-    const int j = (mype + s) % npes;
-    if (causal && j > mype) continue;
-    items.push_back(make_item(0, c, d.start[j], d.start[j + 1] - d.start[j], (causal && j == mype) ? 0 : -1, (int)items.size()));
-  }
-  const int n_parts = (int)items.size();
   // per-call scratch, like the reference's per-call allocations (:383-394) but freed
-  float* ws = nullptr;
-  const size_t table_bytes = (size_t)n_parts * sizeof(ringattn::WorkItem);
-  const size_t lse_floats = ((size_t)(n_parts + 1) * c + 7) & ~(size_t)7;  // keeps the item table 32-byte aligned
-  RA_HIP(hipMalloc((void**)&ws, ((size_t)n_parts * c * dim + lse_floats) * sizeof(float) + table_bytes));
-  float* o_parts = ws;
-  float* lse_parts = ws + (size_t)n_parts * c * dim;
-  float* lse_tmp = lse_parts + (size_t)n_parts * c;
-  ringattn::WorkItem* d_items = (ringattn::WorkItem*)(lse_parts + lse_floats);
-  hipError_t e = hipMemcpy(d_items, items.data(), table_bytes, hipMemcpyHostToDevice);
-  if (e != hipSuccess) rc = hip_fail(e);
-  if (rc == RINGATTN_OK) {
-    ringattn::BlockStepArgs a;
-    fill_geometry(a, p, d);
-    a.q = q;
-    a.k = k;
-    a.v = v;
-    a.o_part = o_parts;
-    a.lse_part = lse_parts;
-    a.items = d_items;
-    a.n_items = n_parts;
-    a.q_tiles_max = (c + ringattn::kBlockM - 1) / ringattn::kBlockM;
-    a.bh_stride = (int64_t)c * dim;
-    a.part_stride_rows = c;
-    a.S = c;
-    e = ringattn::launch_block_step(a, dtype, dim, nullptr);
-    if (e != hipSuccess) rc = hip_fail(e);
-  }
-  if (rc == RINGATTN_OK) rc = ringattn_merge(o_parts, lse_parts, n_parts, (int64_t)c, dim, dtype, out, lse ? lse : lse_tmp, nullptr);
-  e = hipDeviceSynchronize();  // blocking, as csrc/ring_attention.cu:721
+  void* ws = nullptr;
+  RA_HIP(hipMalloc(&ws, rc_.scratch_bytes));
+  rc = run_rank_call(rc_, ws, q, k, v, out, lse, nullptr);
+  hipError_t e = hipDeviceSynchronize();  // blocking, as csrc/ring_attention.cu:721
   if (rc == RINGATTN_OK && e != hipSuccess) rc = hip_fail(e);
   (void)hipFree(ws);
   return rc;
+}
+
+size_t ringattn_noalloc_scratch_bytes(void) { return kScratchBytes; }
+
+int ringattn_ring_attention_noalloc(const void* q, const void* k, const void* v, void* out, float* lse,
+                                    int npes, int mype, const int* seqlen, int dim, int max_seq,
+                                    int dtype, int causal, float softmax_scale, void* stream) {
+  RankCall rc_;
+  int rc = prepare_rank_call(&rc_, q, k, v, out, npes, mype, seqlen, dim, max_seq, dtype, causal, softmax_scale);
+  if (rc != RINGATTN_OK) return rc;
+  if (rc_.scratch_bytes > kScratchBytes) return RINGATTN_ERR_WORKSPACE;
+  void* base = nullptr;
+  rc = device_scratch(&base);
+  if (rc != RINGATTN_OK) return rc;
+  return run_rank_call(rc_, base, q, k, v, out, lse, (hipStream_t)stream);
 }
 
 const char* ringattn_strerror(int code) {

@@ -62,8 +62,16 @@ struct MergeArgs {
   int half_partials;
 };
 
+// Up to kMaxParts work items passed BY VALUE to a small kernel that writes them to device
+// memory: an item table for callers that may not copy from the host (no allocation, no
+// memcpy node: a plain kernel launch).
+struct ItemPack {
+  WorkItem items[kMaxParts];
+};
+
 // dtype: 0 = fp16, 1 = bf16.  Return hipSuccess or the launch error.
 hipError_t launch_block_step(const BlockStepArgs& a, int dtype, int dim, hipStream_t stream);
 hipError_t launch_merge(const MergeArgs& a, int dtype, int dim, hipStream_t stream);
+hipError_t launch_write_items(const ItemPack& pack, int n, WorkItem* dst, hipStream_t stream);
 
 }  // namespace ringattn

@@ -613,6 +613,12 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
   if (c8 == 0) a.lse[row] = (mx == -INFINITY) ? -INFINITY : mx + __logf(wsum);
 }
 
+// ---- item table from kernel arguments ------------------------------------------------
+__global__ __launch_bounds__(64) void write_items_kernel(const ItemPack pack, int n, WorkItem* dst) {
+  const int i = threadIdx.x;
+  if (i < n) dst[i] = pack.items[i];
+}
+
 // ---- host launchers -----------------------------------------------------------------
 hipError_t launch_block_step(const BlockStepArgs& a, int dtype, int dim, hipStream_t stream) {
   if (a.n_items <= 0) return hipSuccess;
@@ -632,6 +638,13 @@ hipError_t launch_block_step(const BlockStepArgs& a, int dtype, int dim, hipStre
   else if (dtype == 1 && dim == 128) RA_LAUNCH_BLOCK(1, 128);
 #undef RA_LAUNCH_BLOCK
   else return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+hipError_t launch_write_items(const ItemPack& pack, int n, WorkItem* dst, hipStream_t stream) {
+  if (n <= 0) return hipSuccess;
+  if (n > kMaxParts) return hipErrorInvalidValue;
+  write_items_kernel<<<1, 64, 0, stream>>>(pack, n, dst);
   return hipGetLastError();
 }
 
