@@ -2,11 +2,11 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4]
 
-A step is one full forward of the workload: every ring step of every virtual rank (a few
-block-attention launches) plus the merges of the per-step partials, with Q/K/V already
-resident in HBM.  Prints one JSON line.  `value` is algorithmic TFLOP/s (4*B*H*d*visible
+A step is one full forward of the workload: every ring step of every virtual rank and the merge
+of the per-step partials (one block-attention launch, the merge fused at the end of each
+workgroup), with Q/K/V already resident in HBM.  Prints one JSON line.  `value` is algorithmic TFLOP/s (4*B*H*d*visible
 (q,k) pairs per forward) over the wall time of K steps; `roofline` prices the
-block-attention launches of the same forward against the dense MFMA peak, each timed by an
+block-attention launch of the same forward against the dense MFMA peak, timed by an
 event pair on the launch stream (a second pass of K forwards on a plan with the timing
 flag); `merge` times the merge kernel alone against HBM bandwidth; `cpu_baseline` is the
 CPU oracle timed on this host on a bounded sample of the same workload's rows.
@@ -23,9 +23,21 @@ sys.path.insert(0, ROOT)
 # Published MI355X dense peaks used for the roofline (not the 2:1-sparsity figures)
 PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0}
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per block-kernel launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
-# see profiles/; None where not measured for that workload.
-MEASURED_TRAFFIC = {"cfg4": 1.541e9}   # 930.4 MB fetched + 610.7 MB written per launch, average over the 4 launches of a forward
+# HBM bytes per block-kernel launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE): workload ->
+# (bytes, summary under profiles/, sha256[:16] of ringattn_kernels.hip when it was measured).  The figure is only
+# printed while the kernel source is still the one that was profiled.
+MEASURED_TRAFFIC = {}
+BASELINE_METRIC = "ring-attn fwd TFLOP/s + % bf16 MFMA peak, S=32K d=128 8-step ring, 1 GPU"
+
+
+def kernel_source_id():
+    import hashlib
+    path = os.path.join(ROOT, "ringattention_amd", "csrc", "ringattn_kernels.hip")
+    try:
+        with open(path, "rb") as f:
+            return hashlib.sha256(f.read()).hexdigest()[:16]
+    except OSError:
+        return None
 
 
 def describe(w):
@@ -53,9 +65,6 @@ def main():
                     help="also time the ring rank by rank on rank-local buffers (one launch per rank and step)")
     ap.add_argument("--per-step", action="store_true", help="also time one block-attention launch per ring step")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the cpu_baseline sample (0 = skip)")
-    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
-                    help="only run a plain device copy of MIB mebibytes a few times and exit: the known-size kernel "
-                         "that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (P virtual ring ranks on one MI355X); use --gpus 1")
@@ -67,14 +76,6 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     torch.cuda.set_device(0)
-    if args.copy_probe > 0:
-        src = torch.empty(args.copy_probe << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
-        dst = torch.empty_like(src)
-        for _ in range(5):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        print(json.dumps({"copy_probe_bytes": args.copy_probe << 20, "copies": 5}))
-        return
     w = WORKLOADS[args.workload]
 
     q, k, v = api.make_qkv_bits(w)
@@ -88,17 +89,24 @@ def main():
     for _ in range(args.warmup):
         plan.forward(qd, kd, vd, out, lse, stream)
     torch.cuda.synchronize()
+    # K steps between two synchronisations on the host clock, and the same K steps between an
+    # event pair on the launch stream (the protocol of the reference harness, csrc/ring_attention.cu:772-783)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    ev0.record(stream)
     for _ in range(args.steps):
         plan.forward(qd, kd, vd, out, lse, stream)
+    ev1.record(stream)
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step_events = ev0.elapsed_time(ev1) / args.steps
     tflops = w.flops / (ms_per_step * 1e-3) / 1e12
 
     bh = w.batch * w.heads
     peak = PEAK_TFLOPS[w.dtype]
-    # ---- block kernel: the same forward on a plan that records an event pair around each of its
-    # block-attention launches, on the stream they are launched on
+    # ---- block kernel: the same forward on a plan that records an event pair around its
+    # block-attention launch, on the stream it is launched on.  The launch is the whole ring (every
+    # step of every rank, the merge of a workgroup's rows fused at its end).
     timed = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=False,
                               layout=args.layout, timing=True, half_partials=w.half_partials)
     timed.forward(qd, kd, vd, out, lse, stream)
@@ -110,10 +118,17 @@ def main():
     n_launch = launch_ms.shape[1]
     avg_launch_ms = float(launch_ms.mean())
     block_tflops = w.flops / n_launch / (avg_launch_ms * 1e-3) / 1e12
+    traffic, traffic_source = None, "not measured for this workload / layout"
+    if args.layout == "contiguous" and w.name in MEASURED_TRAFFIC:
+        t_bytes, t_profile, t_src = MEASURED_TRAFFIC[w.name]
+        if t_src == kernel_source_id():
+            traffic, traffic_source = t_bytes, t_profile
+        else:
+            traffic_source = f"stale: {t_profile} was measured on kernel source {t_src}, this is {kernel_source_id()}"
     roofline = {
         "kernel": "block_attention_kernel", "bound": "mfma",
         "achieved": round(block_tflops, 2), "peak": peak, "unit": "TFLOP/s", "frac": round(block_tflops / peak, 4),
-        "traffic": MEASURED_TRAFFIC.get(w.name) if args.layout == "contiguous" else None,
+        "traffic": traffic, "traffic_source": traffic_source,
         "launches_per_step": n_launch, "avg_launch_ms": round(avg_launch_ms, 4),
         "avg_launch_flop": w.flops / n_launch,
         "launch_ms": [round(float(x), 4) for x in launch_ms.mean(axis=0)],
@@ -140,7 +155,7 @@ def main():
     merge_bytes = bh * sum(ln * (bin(act).count("1") * part_row + 2 * w.dim + 4) for _, ln, act in eager.merge_regions())
     merge = {"kernel": "merge_kernel", "bound": "hbm", "achieved": round(merge_bytes / (merge_ms * 1e-3) / 1e9, 1),
              "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(merge_bytes / (merge_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-             "ms": round(merge_ms, 4), "bytes": merge_bytes, "launches": len(eager.merge_regions())}
+             "ms": round(merge_ms, 4), "bytes": merge_bytes, "launches": 1, "regions": len(eager.merge_regions())}
 
     # ---- optional: one launch per ring step (what ringattn_block_fwd runs), to show how the work
     # spreads over the steps of the ring
@@ -226,9 +241,10 @@ def main():
                          f"full forward extrapolates to {w.flops / (fl / dt):.0f} s"}
 
     print(json.dumps({
-        "metric": "ring-attn fwd TFLOP/s + % bf16 MFMA peak, S=32K d=128 8-step ring, 1 GPU",
+        "metric": BASELINE_METRIC if (w.name == "cfg4" and args.layout == "contiguous")
+        else f"ring-attn fwd TFLOP/s + % {w.dtype} MFMA peak, {describe(w)}, {args.layout} layout, 1 GPU",
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 4), "ms_per_step_events": round(ms_per_step_events, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w.dtype, "data": "synthetic",
         "config": {"workload": describe(w), "algorithmic_flop": w.flops, "graph": bool(w.graph), "layout": args.layout,
                    "partials": "fp16" if w.half_partials else "fp32"},

@@ -94,9 +94,11 @@ typedef struct ringattn_params {
 
 typedef struct ringattn_plan ringattn_plan;
 
-/* Bytes of device workspace a plan needs (per-step partial O and LSE for every ring
- * step): npes * batch*heads*S * (dim + 1) * 4, or npes * batch*heads*S * (2 dim + 4) with
- * RINGATTN_FLAG_HALF_PARTIALS.  0 if the parameters are invalid. */
+/* Bytes of device workspace a plan needs: one partial O row and one partial LSE per query row
+ * and VISIBLE ring step -- (dim + 1) * 4 bytes each, (2 dim + 4) with RINGATTN_FLAG_HALF_PARTIALS.
+ * Without a mask every row has npes steps; with the causal mask a row of rank r has r + 1 (36 of
+ * the 64 (rank, step) pairs at npes = 8); with the zigzag layout the low half of rank r has r + 1
+ * and the high half npes.  0 if the parameters are invalid. */
 size_t ringattn_workspace_bytes(const ringattn_params* params);
 
 /*
@@ -114,9 +116,9 @@ int ringattn_plan_destroy(ringattn_plan* plan);
 
 /*
  * The whole forward for all npes virtual ranks: replaces ring_attention()
- * (csrc/ring_attention.cu:706-722) run on every PE.  Every ring step of every rank (a few
- * block-attention launches that each hold all steps of some ranks), then the merge of each
- * rank's per-step partials, overlapped with the next launch on an internal stream.
+ * (csrc/ring_attention.cu:706-722) run on every PE.  ONE block-attention launch: a workgroup
+ * owns 128 query rows, walks every ring step of those rows like the reference's CTA
+ * (:439-443,456), writes a partial (O, LSE) per step into the workspace and merges them.
  *   q, k, v : [batch, heads, S, dim] dtype     out : same shape and dtype
  *   lse     : [batch, heads, S] fp32, natural log (the reference never writes it)
  * Asynchronous on `stream` (a hipStream_t, or NULL for the default stream); the
@@ -194,7 +196,9 @@ int ringattn_rank_merge(ringattn_plan* plan, int rank, const void* o_parts, cons
  * (local to the KV range) is visible to query ql (local to the query range) iff
  * kl <= ql + diag_off.  The partial result goes to slot `slot` (= the ring step).
  * step in [0, npes): the items ringattn_block_fwd(step) runs; step == -1: all items of
- * ringattn_fwd in launch order.  Writes min(n, capacity) items and stores n in *n_out.
+ * ringattn_fwd, row range by row range, in the order a workgroup runs them (a range that is
+ * masked differently within a rank, as the two halves of a zigzag rank are, is listed as
+ * separate items).  Writes min(n, capacity) items and stores n in *n_out.
  */
 typedef struct ringattn_work_item {
   int q_start, q_len, kv_start, kv_len, diag_off, slot;
@@ -203,11 +207,11 @@ typedef struct ringattn_work_item {
 int ringattn_plan_work_items(const ringattn_plan* plan, int step, ringattn_work_item* out, int capacity, int* n_out);
 
 /*
- * Durations in milliseconds of the block-attention launches of the most recent ringattn_fwd
- * on a plan created with RINGATTN_FLAG_TIMING, from events recorded on the caller's stream
- * right before and after each launch -- the job of the cudaEvent pair around the timed loop
- * of the reference harness (csrc/ring_attention.cu:772-783), per launch.  Blocks until that
- * forward's launches have finished.  Writes min(n, capacity) values and stores n in *n_out;
+ * Durations in milliseconds of the block-attention launches (one, as things are) of the most
+ * recent ringattn_fwd on a plan created with RINGATTN_FLAG_TIMING, from events recorded on the
+ * caller's stream right before and after each launch -- the job of the cudaEvent pair around the
+ * timed loop of the reference harness (csrc/ring_attention.cu:772-783), per launch.  Blocks until
+ * that forward's launches have finished.  Writes min(n, capacity) values and stores n in *n_out;
  * RINGATTN_ERR_PLAN if the plan has no timing flag or has not run a forward yet.
  */
 int ringattn_plan_launch_times(ringattn_plan* plan, float* ms, int capacity, int* n_out);
@@ -240,10 +244,10 @@ int ringattn_ring_attention(const void* q, const void* k, const void* v, void* o
  * reference (whose entry allocates on every call, csrc/ring_attention.cu:383-394).  Same
  * arguments and results as ringattn_ring_attention, plus the stream; it calls no hipMalloc,
  * hipFree, memcpy or other allocating routine and does not synchronise: the work (a
- * table-writing kernel, the block kernel, the merge) is queued on `stream`.  The per-step
+ * table-writing kernel, then the block kernel with its fused merge) is queued on `stream`.  The per-step
  * partials live in a static device array of ringattn_noalloc_scratch_bytes() bytes (32 MiB,
  * held by every GPU the library runs on until the process ends); a call that needs more --
- * visible_steps * (seqlen[mype] * (dim + 1) * 4 + 32) + seqlen[mype] * 4 bytes, visible_steps
+ * visible_steps * (seqlen[mype] * (dim + 1) * 4 + 32) + seqlen[mype] * 4 + 64 bytes, visible_steps
  * being npes, or mype + 1 with the causal mask -- returns RINGATTN_ERR_WORKSPACE.  All calls on
  * one GPU share that array: calls that overlap on one GPU (two streams, two threads) race;
  * nothing in it needs clearing between calls.

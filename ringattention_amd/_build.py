@@ -15,7 +15,7 @@ SOURCES = ["ringattn_kernels.hip", "ringattn_api.hip", "ringattn_datagen.cpp"]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-pthread",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-pthread", "-Wno-inline-asm",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 

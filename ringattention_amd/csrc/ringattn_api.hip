@@ -5,6 +5,7 @@
 #include "ringattn.h"
 #include "ringattn_kernels.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -32,7 +33,6 @@ inline int hip_fail(hipError_t e) {
     if (e__ != hipSuccess) return hip_fail(e__); \
   } while (0)
 
-constexpr int kMaxGroups = 8;  // block launches per forward
 constexpr float kLog2e = 1.4426950408889634f;
 
 struct Derived {
@@ -92,12 +92,6 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 inline bool half_partials(const ringattn_params& p) { return (p.flags & RINGATTN_FLAG_HALF_PARTIALS) != 0; }
 
-// partial O of every slot (fp32, or fp16 with RINGATTN_FLAG_HALF_PARTIALS), then the fp32 partial LSEs
-size_t workspace_bytes_of(const ringattn_params* p, const Derived& d) {
-  const size_t o_elem = half_partials(*p) ? 2 : 4;
-  return (size_t)p->npes * (size_t)d.rows * ((size_t)p->dim * o_elem + sizeof(float));
-}
-
 inline ringattn::WorkItem make_item(int q_start, int q_len, int kv_start, int kv_len, int diag_off, int slot) {
   ringattn::WorkItem w;
   w.q_start = q_start;
@@ -136,18 +130,78 @@ void append_items(std::vector<ringattn::WorkItem>& out, const Derived& d, int P,
   }
 }
 
-}  // namespace
-
-// One block launch of the forward: all ring steps of a few virtual ranks.
-struct LaunchGroup {
-  int item_begin, item_count;      // slice of the item table
-  int region_begin, region_count;  // slice of `regions`: what is merged after this launch
+// A SEGMENT: rows of one rank that meet the same ring steps, with those steps' key ranges in
+// ascending step order -- what one workgroup of the block kernel walks (the reference's CTA
+// walks the steps of its rows the same way, csrc/ring_attention.cu:456-620).  Contiguous
+// layouts have one segment per rank; a zigzag rank has two (its low half sees fewer steps).
+struct HostSegment {
+  int start = 0, len = 0;
+  std::vector<ringattn::WorkItem> items;  // restricted to the segment: q_start = start, q_len = len
+  uint64_t active = 0;                    // the steps (partial slots) of the items
+  int64_t tile_work = 0;                  // keys the busiest 128-row tile of the segment visits
 };
 
-// Rows [start, start + len) of every head share one set of active partial slots.
-struct MergeRegion {
-  int start, len;
-  uint64_t active;
+void rank_segments(std::vector<HostSegment>& out, const Derived& d, int P, bool causal, int r) {
+  std::vector<ringattn::WorkItem> all;
+  for (int s = 0; s < P; ++s) append_items(all, d, P, causal, r, s);
+  const int q0 = d.start[r], q1 = d.start[r + 1];
+  std::vector<int> cut{q0, q1};
+  if (d.zigzag) cut.push_back(q0 + (q1 - q0) / 2);
+  for (const auto& w : all) {
+    cut.push_back(w.q_start);
+    cut.push_back(w.q_start + w.q_len);
+  }
+  std::sort(cut.begin(), cut.end());
+  cut.erase(std::unique(cut.begin(), cut.end()), cut.end());
+  for (size_t i = 0; i + 1 < cut.size(); ++i) {
+    HostSegment sg;
+    sg.start = cut[i];
+    sg.len = cut[i + 1] - cut[i];
+    for (const auto& w : all) {
+      if (w.q_start > sg.start || sg.start + sg.len > w.q_start + w.q_len) continue;
+      ringattn::WorkItem x = w;
+      x.q_start = sg.start;
+      x.q_len = sg.len;
+      if (w.diag_off >= 0) x.diag_off = w.diag_off + (sg.start - w.q_start);
+      sg.items.push_back(x);
+      sg.active |= (uint64_t)1 << w.slot;
+      sg.tile_work += x.diag_off >= 0 ? std::min<int64_t>(x.kv_len, (int64_t)x.diag_off + sg.len) : x.kv_len;
+    }
+    if (!sg.items.empty()) out.push_back(sg);
+  }
+}
+
+// All segments of a forward, busiest first: the block kernel's workgroups are dispatched in
+// this order, so the launch ends on its shortest ones.
+std::vector<HostSegment> forward_segments(const Derived& d, int P, bool causal) {
+  std::vector<HostSegment> segs;
+  for (int r = 0; r < P; ++r) rank_segments(segs, d, P, causal, r);
+  std::stable_sort(segs.begin(), segs.end(),
+                   [](const HostSegment& x, const HostSegment& y) { return x.tile_work > y.tile_work; });
+  return segs;
+}
+
+// Workspace of a forward: one partial block [batch*heads, len] rows per (segment, item) --
+// only the (rank, step) pairs the mask leaves visible -- partial O of every block first (fp32,
+// or fp16 with RINGATTN_FLAG_HALF_PARTIALS), then the fp32 partial LSEs.
+int64_t partial_rows_of(const std::vector<HostSegment>& segs, const Derived& d) {
+  int64_t rows = 0;
+  for (const auto& sg : segs) rows += (int64_t)sg.items.size() * d.BH * sg.len;
+  return rows;
+}
+
+size_t workspace_bytes_of(const ringattn_params* p, const Derived& d) {
+  const size_t o_elem = half_partials(*p) ? 2 : 4;
+  const int64_t rows = partial_rows_of(forward_segments(d, p->npes, p->causal != 0), d);
+  return (size_t)rows * ((size_t)p->dim * o_elem + sizeof(float));
+}
+
+}  // namespace
+
+// A slice of the device tables: what one block launch runs.
+struct TableSlice {
+  int seg_begin = 0, seg_count = 0;
+  int q_tiles_max = 0;
 };
 
 struct ringattn_plan {
@@ -157,29 +211,36 @@ struct ringattn_plan {
   void* ws = nullptr;
   size_t ws_bytes = 0;
   bool own_ws = false;
-  void* o_parts = nullptr;     // [npes, rows, dim] fp32 (fp16 with RINGATTN_FLAG_HALF_PARTIALS)
-  float* lse_parts = nullptr;  // [npes, rows]
-  // Item table (host copy + device copy made at the first forward): first the launch
-  // schedule of ringattn_fwd, then one list per ring step for ringattn_block_fwd.
-  // The ring steps of different ranks are independent (each item writes its own rows of its
-  // step's partial slot), so the forward is issued as a few launches that each hold ALL
-  // steps of a few ranks; the merge of those ranks then runs on a second stream underneath
-  // the next launch.
+  void* o_parts = nullptr;     // partial O rows, fp32 (fp16 with RINGATTN_FLAG_HALF_PARTIALS)
+  float* lse_parts = nullptr;  // partial LSE rows
+  // Segment / item tables (host copies + device copies made at the first launch).  Three
+  // families of slices: the forward (all ring steps of every rank, one launch, partials in the
+  // workspace), one ring step of every rank (ringattn_block_fwd, partials in the caller's
+  // [batch*heads, S] slot), one step of one rank on rank-local rows (ringattn_rank_step_fwd).
+  std::vector<ringattn::Segment> h_segs;
+  std::vector<ringattn::SegItem> h_segitems;
+  TableSlice fwd;
+  std::vector<TableSlice> step;    // [npes]
+  std::vector<TableSlice> local;   // [npes * npes]
+  // the same schedule as plain work items, for ringattn_plan_work_items
   std::vector<ringattn::WorkItem> h_items;
-  std::vector<LaunchGroup> groups;
-  std::vector<MergeRegion> regions;  // group by group, then (from all_regions on) rank by rank
-  int all_regions = 0;
-  std::vector<int> step_begin;       // [npes + 1] slices of h_items, one per ring step
-  std::vector<int> local_begin;      // [npes * npes + 1] slices of h_items: the items of (rank, step) in
-                                     // rank-local rows (queries from 0, keys from 0 of the visited chunk)
-  int q_tiles_max = 0;
-  ringattn::WorkItem* d_items = nullptr;
-  hipStream_t merge_stream = nullptr;
-  hipEvent_t ev_group[kMaxGroups]{};
-  hipEvent_t ev_done = nullptr;
-  hipEvent_t ev_t0[kMaxGroups]{}, ev_t1[kMaxGroups]{};  // RINGATTN_FLAG_TIMING: around each block launch
-  bool timed_forward = false;                            // a forward has recorded them
-  bool streams_ready = false;
+  int fwd_items = 0;               // h_items[0, fwd_items): the forward, in run order
+  std::vector<int> step_begin;     // [npes + 1] slices of h_items, one per ring step
+  // merge regions, rank by rank (global rows), then the same with rank-local rows
+  std::vector<ringattn::MergeRegion> regions;
+  int n_regions = 0;               // global ones; regions[n_regions + i] is regions[i] in local rows
+  std::vector<int> region_rank;    // [n_regions]
+  int region_max_len = 0;
+  // forward only: per XCD, the (segment, head) pairs its workgroups run, heads dealt round-robin
+  std::vector<int2> fwd_groups;
+  int fwd_groups_per_xcd = 0;
+  int2* d_groups = nullptr;
+  ringattn::Segment* d_segs = nullptr;
+  ringattn::SegItem* d_segitems = nullptr;
+  ringattn::MergeRegion* d_regions = nullptr;
+  hipEvent_t ev_t0 = nullptr, ev_t1 = nullptr;  // RINGATTN_FLAG_TIMING: around the block launch
+  bool timed_forward = false;                    // a forward has recorded them
+  bool tables_ready = false;
   // hipGraph replay (RINGATTN_FLAG_GRAPH): one captured graph per pointer set
   hipStream_t cap_stream = nullptr;
   hipGraph_t graph = nullptr;
@@ -192,12 +253,11 @@ struct ringattn_plan {
 namespace {
 
 // fields of the launch arguments that depend only on the geometry
-void fill_geometry(ringattn::BlockStepArgs& a, const ringattn_params& p, const Derived& d) {
+void fill_geometry(ringattn::BlockArgs& a, const ringattn_params& p, const Derived& d) {
+  std::memset(&a, 0, sizeof(a));
   a.bh_stride = d.S * p.dim;
   a.kv_bh_stride = d.S * p.dim;
-  a.part_stride_rows = d.rows;
   a.S = (int)d.S;
-  a.slot_bias = 0;
   a.BH = (int)d.BH;
   a.heads = p.heads;
   a.kv_group = p.kv_heads > 0 ? p.heads / p.kv_heads : 1;
@@ -205,198 +265,197 @@ void fill_geometry(ringattn::BlockStepArgs& a, const ringattn_params& p, const D
   a.half_partials = half_partials(p) ? 1 : 0;
 }
 
-// The rows of rank r that share a set of active slots, with that set: slot s is active for
-// a row iff the item list of (r, s) covers the row.
-void append_regions(std::vector<MergeRegion>& out, const Derived& d, int P, bool causal, int r) {
-  const int q0 = d.start[r], ql = d.start[r + 1] - q0;
-  const int parts = d.zigzag ? 2 : 1;
-  for (int i = 0; i < parts; ++i) {
-    MergeRegion m;
-    m.start = q0 + i * (ql / parts);
-    m.len = ql / parts;
-    m.active = 0;
-    std::vector<ringattn::WorkItem> items;
-    for (int s = 0; s < P; ++s) {
-      items.clear();
-      append_items(items, d, P, causal, r, s);
-      for (const auto& w : items)
-        if (w.q_start <= m.start && m.start + m.len <= w.q_start + w.q_len) m.active |= (uint64_t)1 << s;
+inline int q_tiles_of(int len) { return (len + ringattn::kBlockM - 1) / ringattn::kBlockM; }
+
+// Appends one segment with its items to the tables.  part_base(i) / stride: where item i's
+// partial block lives.  A masked (diagonal) item runs last and the q tiles go busiest first.
+template <class BaseFn>
+void push_segment(ringattn_plan* pl, TableSlice& slice, int q_start, int q_len,
+                  const std::vector<ringattn::WorkItem>& items, int kv_shift, BaseFn part_base, int part_bh_stride) {
+  ringattn::Segment sg;
+  std::memset(&sg, 0, sizeof(sg));
+  sg.q_start = q_start;
+  sg.q_len = q_len;
+  sg.item_begin = (int)pl->h_segitems.size();
+  sg.item_count = (int)items.size();
+  sg.last_item = -1;
+  for (size_t i = 0; i < items.size(); ++i) {
+    const ringattn::WorkItem& w = items[i];
+    ringattn::SegItem it;
+    std::memset(&it, 0, sizeof(it));
+    it.kv_start = w.kv_start - kv_shift;
+    it.kv_len = w.kv_len;
+    it.diag_off = w.diag_off;
+    it.part_bh_stride = part_bh_stride;
+    it.part_base = part_base((int)i);
+    it.slot = w.slot;
+    if (w.diag_off >= 0) {
+      sg.last_item = (int)i;
+      sg.reverse_tiles = 1;
     }
-    out.push_back(m);
+    pl->h_segitems.push_back(it);
   }
+  if (sg.item_count == 1) sg.last_item = -1;
+  pl->h_segs.push_back(sg);
+  ++slice.seg_count;
+  slice.q_tiles_max = std::max(slice.q_tiles_max, q_tiles_of(q_len));
 }
 
-// Launch schedule.  Contiguous causal: rank r has r + 1 visible chunks, so ranks are paired
-// (P-1-g, g) to give every launch the same work; otherwise (no mask, or zigzag, where all
-// ranks have equal work) consecutive ranks.  At most kMaxGroups launches.  Within a launch
-// the items of one rank are listed in ring order.
+// The tables of a plan (host side; nothing here touches the GPU).
 void build_schedule(ringattn_plan* pl) {
   const int P = pl->p.npes;
   const Derived& d = pl->d;
   const bool causal = pl->p.causal != 0;
-  const bool paired = causal && !d.zigzag;
-  std::vector<int> order;  // ranks in launch order
-  if (paired) {
-    for (int g = 0; g < (P + 1) / 2; ++g) {
-      order.push_back(P - 1 - g);
-      if (g != P - 1 - g) order.push_back(g);
+
+  // ---- the forward: every segment with all its steps; partial blocks packed in the workspace
+  const std::vector<HostSegment> segs = forward_segments(d, P, causal);
+  pl->fwd.seg_begin = 0;
+  int64_t next_row = 0;
+  for (const auto& sg : segs) {
+    const int64_t block_rows = d.BH * sg.len;
+    const int64_t base = next_row;
+    push_segment(pl, pl->fwd, sg.start, sg.len, sg.items, 0,
+                 [&](int i) { return base + (int64_t)i * block_rows; }, sg.len);
+    next_row += (int64_t)sg.items.size() * block_rows;
+    // the same items in run order (the masked one last), for inspection
+    const ringattn::Segment& t = pl->h_segs.back();
+    for (int i = 0; i < t.item_count; ++i) {
+      int idx = i;
+      if (t.last_item >= 0) idx = (i == t.item_count - 1) ? t.last_item : (i >= t.last_item ? i + 1 : i);
+      pl->h_items.push_back(sg.items[(size_t)idx]);
     }
-  } else if (d.zigzag) {
-    // rank 0 merges the fewest partials: last, where the merge is not hidden under a launch
-    for (int r = P - 1; r >= 0; --r) order.push_back(r);
-  } else {
-    for (int r = 0; r < P; ++r) order.push_back(r);
   }
-  int n_groups;
-  if (P < 4) n_groups = 1;
-  else if (paired) n_groups = (P + 1) / 2 < kMaxGroups ? (P + 1) / 2 : kMaxGroups;
-  else n_groups = P < 8 ? P / 2 : 4;
-  {
-    // Splitting only pays when every launch still fills the chip many times over: count the
-    // workgroups of the whole forward (128 query rows each) and keep at least 4096 per launch
-    // (8 rounds of 2 workgroups on each of 256 CUs).
-    std::vector<ringattn::WorkItem> all;
-    for (int r = 0; r < P; ++r)
-      for (int s = 0; s < P; ++s) append_items(all, d, P, causal, r, s);
-    int64_t wgs = 0;
-    for (const auto& w : all) wgs += (w.q_len + ringattn::kBlockM - 1) / ringattn::kBlockM;
-    wgs *= d.BH;
-    const int64_t fit = wgs / 4096;
-    if (fit < n_groups) n_groups = fit < 1 ? 1 : (int)fit;
-  }
-  size_t pos = 0;
-  for (int g = 0; g < n_groups; ++g) {
-    // even split of the rank list; paired lists come in balanced pairs, keep pairs together
-    size_t end = order.size() * (size_t)(g + 1) / (size_t)n_groups;
-    if (paired && (end & 1) && end < order.size()) ++end;
-    if (g == n_groups - 1) end = order.size();
-    if (end <= pos) continue;
-    LaunchGroup lg;
-    lg.item_begin = (int)pl->h_items.size();
-    lg.region_begin = (int)pl->regions.size();
-    for (size_t i = pos; i < end; ++i) {
-      const int r = order[i];
-      append_regions(pl->regions, d, P, causal, r);
-      for (int s = 0; s < P; ++s) append_items(pl->h_items, d, P, causal, r, s);
+  pl->fwd_items = (int)pl->h_items.size();
+  // Workgroup order of the forward.  Heads are dealt to the 8 XCDs round-robin; an XCD runs
+  // the segments of one head after the other (busiest first within a head), so the ranks of
+  // a head, which read the same K and V, follow each other through that XCD's L2.  Only when
+  // the heads divide evenly; otherwise the kernel's arithmetic mapping spreads (segment,
+  // head) pairs over the XCDs.
+  if (d.BH % 8 == 0) {
+    const int heads_per_xcd = (int)(d.BH / 8);
+    pl->fwd_groups_per_xcd = heads_per_xcd * pl->fwd.seg_count;
+    pl->fwd_groups.assign((size_t)8 * pl->fwd_groups_per_xcd, int2{-1, -1});
+    for (int x = 0; x < 8; ++x) {
+      size_t pos = (size_t)x * pl->fwd_groups_per_xcd;
+      for (int hh = 0; hh < heads_per_xcd; ++hh)
+        for (int sgi = 0; sgi < pl->fwd.seg_count; ++sgi) pl->fwd_groups[pos++] = int2{sgi, hh * 8 + x};
     }
-    lg.item_count = (int)pl->h_items.size() - lg.item_begin;
-    lg.region_count = (int)pl->regions.size() - lg.region_begin;
-    pl->groups.push_back(lg);
-    pos = end;
   }
-  pl->all_regions = (int)pl->regions.size();
-  for (int r = 0; r < P; ++r) append_regions(pl->regions, d, P, causal, r);
-  // per-step lists: one ring step of every rank
+
+  // ---- one ring step of every rank: partials at the rows of the queries in a [BH, S] slot
   for (int s = 0; s < P; ++s) {
     pl->step_begin.push_back((int)pl->h_items.size());
-    for (int r = 0; r < P; ++r) append_items(pl->h_items, d, P, causal, r, s);
-  }
-  pl->step_begin.push_back((int)pl->h_items.size());
-  // rank-local lists for ringattn_rank_step_fwd: one (rank, step) at a time, rows counted from the
-  // start of the rank's own chunk and of the visited chunk, one partial slot
-  for (int r = 0; r < P; ++r)
-    for (int s = 0; s < P; ++s) {
-      pl->local_begin.push_back((int)pl->h_items.size());
-      const size_t first = pl->h_items.size();
-      append_items(pl->h_items, d, P, causal, r, s);
-      for (size_t i = first; i < pl->h_items.size(); ++i) {
-        pl->h_items[i].q_start -= d.start[r];
-        pl->h_items[i].kv_start -= d.start[(r + s) % P];
-        pl->h_items[i].slot = 0;
+    TableSlice sl;
+    sl.seg_begin = (int)pl->h_segs.size();
+    std::vector<ringattn::WorkItem> one;
+    for (int r = 0; r < P; ++r) {
+      one.clear();
+      append_items(one, d, P, causal, r, s);
+      for (const auto& w : one) {
+        pl->h_items.push_back(w);
+        const std::vector<ringattn::WorkItem> v1{w};
+        push_segment(pl, sl, w.q_start, w.q_len, v1, 0, [&](int) { return (int64_t)w.q_start; }, (int)d.S);
       }
     }
-  pl->local_begin.push_back((int)pl->h_items.size());
-  int longest = 0;
-  for (const auto& w : pl->h_items) longest = w.q_len > longest ? w.q_len : longest;
-  pl->q_tiles_max = (longest + ringattn::kBlockM - 1) / ringattn::kBlockM;
+    pl->step.push_back(sl);
+  }
+  pl->step_begin.push_back((int)pl->h_items.size());
+
+  // ---- one step of one rank in rank-local rows (queries from 0, keys from 0 of the visited chunk)
+  for (int r = 0; r < P; ++r)
+    for (int s = 0; s < P; ++s) {
+      TableSlice sl;
+      sl.seg_begin = (int)pl->h_segs.size();
+      std::vector<ringattn::WorkItem> one;
+      append_items(one, d, P, causal, r, s);
+      const int q0 = d.start[r], rows = d.start[r + 1] - q0, k0 = d.start[(r + s) % P];
+      for (const auto& w : one) {
+        const std::vector<ringattn::WorkItem> v1{w};
+        push_segment(pl, sl, w.q_start - q0, w.q_len, v1, k0, [&](int) { return (int64_t)(w.q_start - q0); }, rows);
+      }
+      pl->local.push_back(sl);
+    }
+
+  // ---- merge regions of caller-held per-step partials, rank by rank
+  for (int r = 0; r < P; ++r) {
+    std::vector<HostSegment> rs;
+    rank_segments(rs, d, P, causal, r);
+    for (const auto& sg : rs) {
+      pl->regions.push_back(ringattn::MergeRegion{sg.start, sg.len, sg.active});
+      pl->region_rank.push_back(r);
+      pl->region_max_len = std::max(pl->region_max_len, sg.len);
+    }
+  }
+  pl->n_regions = (int)pl->regions.size();
+  for (int i = 0; i < pl->n_regions; ++i) {
+    ringattn::MergeRegion m = pl->regions[(size_t)i];
+    m.start -= d.start[pl->region_rank[(size_t)i]];
+    pl->regions.push_back(m);
+  }
 }
 
-int ensure_streams(ringattn_plan* pl) {
-  if (pl->streams_ready) return RINGATTN_OK;
+// Device copies of the tables and the timing events: made at the first launch, outside any capture.
+int ensure_tables(ringattn_plan* pl) {
+  if (pl->tables_ready) return RINGATTN_OK;
   // a call that failed half way is resumed: nothing is created twice
-  const size_t bytes = pl->h_items.size() * sizeof(ringattn::WorkItem);
-  if (!pl->d_items) RA_HIP(hipMalloc((void**)&pl->d_items, bytes));
-  RA_HIP(hipMemcpy(pl->d_items, pl->h_items.data(), bytes, hipMemcpyHostToDevice));
-  if (!pl->merge_stream) RA_HIP(hipStreamCreateWithFlags(&pl->merge_stream, hipStreamNonBlocking));
-  for (int i = 0; i < kMaxGroups; ++i)
-    if (!pl->ev_group[i]) RA_HIP(hipEventCreateWithFlags(&pl->ev_group[i], hipEventDisableTiming));
-  if (!pl->ev_done) RA_HIP(hipEventCreateWithFlags(&pl->ev_done, hipEventDisableTiming));
-  if (pl->p.flags & RINGATTN_FLAG_TIMING)
-    for (int i = 0; i < kMaxGroups; ++i) {
-      if (!pl->ev_t0[i]) RA_HIP(hipEventCreate(&pl->ev_t0[i]));
-      if (!pl->ev_t1[i]) RA_HIP(hipEventCreate(&pl->ev_t1[i]));
-    }
-  pl->streams_ready = true;
+  const size_t seg_bytes = pl->h_segs.size() * sizeof(ringattn::Segment);
+  const size_t item_bytes = pl->h_segitems.size() * sizeof(ringattn::SegItem);
+  const size_t reg_bytes = pl->regions.size() * sizeof(ringattn::MergeRegion);
+  if (!pl->d_segs) RA_HIP(hipMalloc((void**)&pl->d_segs, seg_bytes));
+  if (!pl->d_segitems) RA_HIP(hipMalloc((void**)&pl->d_segitems, item_bytes));
+  if (!pl->d_regions) RA_HIP(hipMalloc((void**)&pl->d_regions, reg_bytes));
+  if (!pl->fwd_groups.empty()) {
+    const size_t grp_bytes = pl->fwd_groups.size() * sizeof(int2);
+    if (!pl->d_groups) RA_HIP(hipMalloc((void**)&pl->d_groups, grp_bytes));
+    RA_HIP(hipMemcpy(pl->d_groups, pl->fwd_groups.data(), grp_bytes, hipMemcpyHostToDevice));
+  }
+  RA_HIP(hipMemcpy(pl->d_segs, pl->h_segs.data(), seg_bytes, hipMemcpyHostToDevice));
+  RA_HIP(hipMemcpy(pl->d_segitems, pl->h_segitems.data(), item_bytes, hipMemcpyHostToDevice));
+  RA_HIP(hipMemcpy(pl->d_regions, pl->regions.data(), reg_bytes, hipMemcpyHostToDevice));
+  if (pl->p.flags & RINGATTN_FLAG_TIMING) {
+    if (!pl->ev_t0) RA_HIP(hipEventCreate(&pl->ev_t0));
+    if (!pl->ev_t1) RA_HIP(hipEventCreate(&pl->ev_t1));
+  }
+  pl->tables_ready = true;
   return RINGATTN_OK;
 }
 
-// A block launch over a slice of the item table; o_part / lse_part: partial slot `slot_bias`.
-int launch_items(const ringattn_plan* pl, int item_begin, int item_count, const void* q, const void* k,
-                 const void* v, void* o_part, float* lse_part, int slot_bias, hipStream_t stream) {
-  ringattn::BlockStepArgs a;
+// A block launch over a slice of the tables.
+int launch_slice(const ringattn_plan* pl, const TableSlice& sl, ringattn::BlockArgs& a, hipStream_t stream) {
+  if (sl.seg_count == 0) return RINGATTN_OK;
+  a.segs = pl->d_segs + sl.seg_begin;
+  a.items = pl->d_segitems;
+  a.n_segs = sl.seg_count;
+  a.q_tiles_max = sl.q_tiles_max;
+  RA_HIP(ringattn::launch_block(a, pl->p.dtype, pl->p.dim, stream));
+  return RINGATTN_OK;
+}
+
+// The ring step loop (csrc/ring_attention.cu:456-620) plus the merge, ONE launch: every
+// workgroup walks the ring steps of its 128 rows, writes a partial (O, LSE) per step and
+// merges them at the end.
+int run_forward(ringattn_plan* pl, const void* q, const void* k, const void* v, void* out,
+                float* lse, hipStream_t stream) {
+  const bool timing = (pl->p.flags & RINGATTN_FLAG_TIMING) && !(pl->p.flags & RINGATTN_FLAG_GRAPH);
+  ringattn::BlockArgs a;
   fill_geometry(a, pl->p, pl->d);
   a.q = q;
   a.k = k;
   a.v = v;
-  a.o_part = o_part;
-  a.lse_part = lse_part;
-  a.items = pl->d_items + item_begin;
-  a.n_items = item_count;
-  a.q_tiles_max = pl->q_tiles_max;
-  a.slot_bias = slot_bias;
-  RA_HIP(ringattn::launch_block_step(a, pl->p.dtype, pl->p.dim, stream));
-  return RINGATTN_OK;
-}
-
-int launch_region_merge(const ringattn_plan* pl, const void* o_parts, const float* lse_parts, void* out,
-                        float* lse, hipStream_t stream, const MergeRegion& reg) {
-  ringattn::MergeArgs m;
-  m.o_parts = o_parts;
-  m.lse_parts = lse_parts;
-  m.out = out;
-  m.lse = lse;
-  m.sel_start = reg.start;
-  m.sel_len = reg.len;
-  m.rows = pl->d.BH * reg.len;
-  m.part_stride_rows = pl->d.rows;
-  m.active = reg.active;
-  m.half_partials = half_partials(pl->p) ? 1 : 0;
-  m.S = (int)pl->d.S;
-  RA_HIP(ringattn::launch_merge(m, pl->p.dtype, pl->p.dim, stream));
-  return RINGATTN_OK;
-}
-
-// The ring step loop (csrc/ring_attention.cu:456-620 moved to the host) plus the merge:
-// for every launch group, all ring steps of its ranks, then the merge of those ranks'
-// rows on the merge stream while the next group computes.  The last group's merge runs
-// on the caller's stream, which finally waits for the merge stream.
-int run_forward(ringattn_plan* pl, const void* q, const void* k, const void* v, void* out,
-                float* lse, hipStream_t stream) {
-  int rc = RINGATTN_OK;
-  const size_t G = pl->groups.size();
-  const bool timing = (pl->p.flags & RINGATTN_FLAG_TIMING) && !(pl->p.flags & RINGATTN_FLAG_GRAPH);
-  for (size_t g = 0; g < G; ++g) {
-    const LaunchGroup& lg = pl->groups[g];
-    if (timing) RA_HIP(hipEventRecord(pl->ev_t0[g], stream));
-    rc = launch_items(pl, lg.item_begin, lg.item_count, q, k, v, pl->o_parts, pl->lse_parts, 0, stream);
-    if (rc != RINGATTN_OK) return rc;
-    if (timing) RA_HIP(hipEventRecord(pl->ev_t1[g], stream));
-    hipStream_t ms = stream;
-    if (g + 1 < G) {
-      RA_HIP(hipEventRecord(pl->ev_group[g], stream));
-      RA_HIP(hipStreamWaitEvent(pl->merge_stream, pl->ev_group[g], 0));
-      ms = pl->merge_stream;
-    }
-    for (int i = 0; i < lg.region_count; ++i) {
-      rc = launch_region_merge(pl, pl->o_parts, pl->lse_parts, out, lse, ms, pl->regions[lg.region_begin + i]);
-      if (rc != RINGATTN_OK) return rc;
-    }
+  a.o_part = pl->o_parts;
+  a.lse_part = pl->lse_parts;
+  a.out = out;
+  a.lse = lse;
+  a.fuse_merge = 1;
+  a.groups = pl->d_groups;
+  a.groups_per_xcd = pl->fwd_groups_per_xcd;
+  if (timing) RA_HIP(hipEventRecord(pl->ev_t0, stream));
+  const int rc = launch_slice(pl, pl->fwd, a, stream);
+  if (rc != RINGATTN_OK) return rc;
+  if (timing) {
+    RA_HIP(hipEventRecord(pl->ev_t1, stream));
+    pl->timed_forward = true;
   }
-  if (G > 1) {
-    RA_HIP(hipEventRecord(pl->ev_done, pl->merge_stream));
-    RA_HIP(hipStreamWaitEvent(stream, pl->ev_done, 0));
-  }
-  if (timing) pl->timed_forward = true;
   return RINGATTN_OK;
 }
 
@@ -413,18 +472,17 @@ inline bool plan_ok(const ringattn_plan* pl) {
   return g_plans.count(pl) != 0;
 }
 
-
 // ---- the reference-shaped call for one rank (ringattn_ring_attention and its variant that
 // allocates nothing) ------------------------------------------------------------------------
 // Device scratch of one call: the rank's per-step partial O [n_parts, c, dim] fp32, partial LSE
-// [n_parts, c], a spare LSE row [c] for callers that pass no lse, and the item table.
+// [n_parts, c], a spare LSE row [c] for callers that pass no lse, and the segment + item table.
 struct RankCall {
   ringattn_params p;
   Derived d;
-  ringattn::ItemPack pack;  // the visible ring steps of the rank in ring order, one compact slot each
+  ringattn::TablePack pack;  // the visible ring steps of the rank in ring order, one compact slot each
   int n_parts = 0;
   int c = 0;                // rows of this rank
-  size_t lse_floats = 0;    // floats of the two LSE areas, padded so the item table stays 32-byte aligned
+  size_t lse_floats = 0;    // floats of the two LSE areas, padded so the table stays 32-byte aligned
   size_t scratch_bytes = 0;
 };
 
@@ -448,46 +506,68 @@ int prepare_rank_call(RankCall* rc, const void* q, const void* k, const void* v,
   if (!q || !k || !v || !out) return RINGATTN_ERR_NULL;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return RINGATTN_ERR_ALIGN;
   // the query rows are local to the caller's rank-sized q and out buffers
-  rc->c = d.start[mype + 1] - d.start[mype];
+  const int c = rc->c = d.start[mype + 1] - d.start[mype];
+  std::memset(&rc->pack, 0, sizeof(rc->pack));
+  ringattn::Segment& sg = rc->pack.seg;
+  sg.q_start = 0;
+  sg.q_len = c;
+  sg.item_begin = 0;
+  sg.last_item = -1;
   rc->n_parts = 0;
   for (int s = 0; s < npes; ++s) {
     const int j = (mype + s) % npes;
     if (causal && j > mype) continue;
-    rc->pack.items[rc->n_parts] =
-        make_item(0, rc->c, d.start[j], d.start[j + 1] - d.start[j], (causal && j == mype) ? 0 : -1, rc->n_parts);
+    ringattn::SegItem& it = rc->pack.items[rc->n_parts];
+    it.kv_start = d.start[j];
+    it.kv_len = d.start[j + 1] - d.start[j];
+    it.diag_off = (causal && j == mype) ? 0 : -1;
+    it.part_bh_stride = c;
+    it.part_base = (int64_t)rc->n_parts * c;
+    it.slot = s;
+    if (it.diag_off >= 0) {
+      sg.last_item = rc->n_parts;
+      sg.reverse_tiles = 1;
+    }
     ++rc->n_parts;
   }
-  rc->lse_floats = ((size_t)(rc->n_parts + 1) * rc->c + 7) & ~(size_t)7;
-  rc->scratch_bytes = ((size_t)rc->n_parts * rc->c * dim + rc->lse_floats) * sizeof(float) +
-                      (size_t)rc->n_parts * sizeof(ringattn::WorkItem);
+  sg.item_count = rc->n_parts;
+  if (rc->n_parts == 1) sg.last_item = -1;
+  rc->lse_floats = ((size_t)(rc->n_parts + 1) * c + 7) & ~(size_t)7;
+  rc->scratch_bytes = ((size_t)rc->n_parts * c * dim + rc->lse_floats) * sizeof(float) + sizeof(ringattn::Segment) +
+                      (size_t)rc->n_parts * sizeof(ringattn::SegItem);
   return RINGATTN_OK;
 }
 
-// Item table (written by a kernel from its arguments), block kernel, merge: three launches on
-// `stream`, nothing is allocated or copied from the host.  `scratch`: rc.scratch_bytes of device memory.
+// The table (written by a kernel from its arguments), then the block kernel with its fused
+// merge: two launches on `stream`, nothing is allocated or copied from the host.
+// `scratch`: rc.scratch_bytes of device memory.
 int run_rank_call(const RankCall& rc, void* scratch, const void* q, const void* k, const void* v, void* out,
                   float* lse, hipStream_t stream) {
   const int dim = rc.p.dim, c = rc.c, n_parts = rc.n_parts;
   float* o_parts = (float*)scratch;
   float* lse_parts = o_parts + (size_t)n_parts * c * dim;
   float* lse_tmp = lse_parts + (size_t)n_parts * c;
-  ringattn::WorkItem* d_items = (ringattn::WorkItem*)(lse_parts + rc.lse_floats);
-  RA_HIP(ringattn::launch_write_items(rc.pack, n_parts, d_items, stream));
-  ringattn::BlockStepArgs a;
+  ringattn::Segment* d_seg = (ringattn::Segment*)(lse_parts + rc.lse_floats);
+  ringattn::SegItem* d_items = (ringattn::SegItem*)(d_seg + 1);
+  RA_HIP(ringattn::launch_write_table(rc.pack, n_parts, d_seg, d_items, stream));
+  ringattn::BlockArgs a;
   fill_geometry(a, rc.p, rc.d);
   a.q = q;
   a.k = k;
   a.v = v;
   a.o_part = o_parts;
   a.lse_part = lse_parts;
+  a.out = out;
+  a.lse = lse ? lse : lse_tmp;
+  a.fuse_merge = 1;
+  a.segs = d_seg;
   a.items = d_items;
-  a.n_items = n_parts;
-  a.q_tiles_max = (c + ringattn::kBlockM - 1) / ringattn::kBlockM;
-  a.bh_stride = (int64_t)c * dim;
-  a.part_stride_rows = c;
+  a.n_segs = 1;
+  a.q_tiles_max = q_tiles_of(c);
+  a.bh_stride = (int64_t)c * dim;  // q and out hold this rank's rows only; k and v the whole sequence
   a.S = c;
-  RA_HIP(ringattn::launch_block_step(a, rc.p.dtype, dim, stream));
-  return ringattn_merge(o_parts, lse_parts, n_parts, (int64_t)c, dim, rc.p.dtype, out, lse ? lse : lse_tmp, stream);
+  RA_HIP(ringattn::launch_block(a, rc.p.dtype, dim, stream));
+  return RINGATTN_OK;
 }
 
 // Static device scratch of ringattn_ring_attention_noalloc.  In host code the array's name is
@@ -511,6 +591,26 @@ int device_scratch(void** base) {
     g_scratch_ptr[dev] = ptr;
   }
   *base = g_scratch_ptr[dev];
+  return RINGATTN_OK;
+}
+
+// merge launch over `count` regions of the plan's device table starting at `first`
+int launch_regions(const ringattn_plan* pl, int first, int count, int max_len, int rows_per_head, int64_t part_stride_rows,
+                   const void* o_parts, const float* lse_parts, void* out, float* lse, hipStream_t stream) {
+  ringattn::MergeArgs m;
+  std::memset(&m, 0, sizeof(m));
+  m.o_parts = o_parts;
+  m.lse_parts = lse_parts;
+  m.out = out;
+  m.lse = lse;
+  m.regions = pl->d_regions + first;
+  m.n_regions = count;
+  m.max_len = max_len;
+  m.heads = (int)pl->d.BH;
+  m.S = rows_per_head;
+  m.part_stride_rows = part_stride_rows;
+  m.half_partials = half_partials(pl->p) ? 1 : 0;
+  RA_HIP(ringattn::launch_merge(m, pl->p.dtype, pl->p.dim, stream));
   return RINGATTN_OK;
 }
 
@@ -555,9 +655,10 @@ int ringattn_plan_create(const ringattn_params* params, void* workspace, size_t 
     }
     pl->own_ws = true;
   }
-  pl->o_parts = pl->ws;
-  pl->lse_parts = (float*)((char*)pl->ws + (size_t)params->npes * d.rows * params->dim * (half_partials(*params) ? 2 : 4));
   build_schedule(pl);
+  const size_t part_rows = need / ((size_t)params->dim * (half_partials(*params) ? 2 : 4) + sizeof(float));
+  pl->o_parts = pl->ws;
+  pl->lse_parts = (float*)((char*)pl->ws + part_rows * params->dim * (half_partials(*params) ? 2 : 4));
   {
     std::lock_guard<std::mutex> lk(g_plans_mu);
     g_plans.insert(pl);
@@ -574,16 +675,13 @@ int ringattn_plan_destroy(ringattn_plan* plan) {
   int rc = RINGATTN_OK;
   drop_graph(plan);
   if (plan->cap_stream) (void)hipStreamDestroy(plan->cap_stream);
-  // whatever ensure_streams() got to create, also after a failure half way
-  if (plan->merge_stream) (void)hipStreamDestroy(plan->merge_stream);
-  for (int i = 0; i < kMaxGroups; ++i)
-    if (plan->ev_group[i]) (void)hipEventDestroy(plan->ev_group[i]);
-  if (plan->ev_done) (void)hipEventDestroy(plan->ev_done);
-  for (int i = 0; i < kMaxGroups; ++i) {
-    if (plan->ev_t0[i]) (void)hipEventDestroy(plan->ev_t0[i]);
-    if (plan->ev_t1[i]) (void)hipEventDestroy(plan->ev_t1[i]);
-  }
-  if (plan->d_items) (void)hipFree(plan->d_items);
+  // whatever ensure_tables() got to create, also after a failure half way
+  if (plan->ev_t0) (void)hipEventDestroy(plan->ev_t0);
+  if (plan->ev_t1) (void)hipEventDestroy(plan->ev_t1);
+  if (plan->d_segs) (void)hipFree(plan->d_segs);
+  if (plan->d_segitems) (void)hipFree(plan->d_segitems);
+  if (plan->d_regions) (void)hipFree(plan->d_regions);
+  if (plan->d_groups) (void)hipFree(plan->d_groups);
   if (plan->own_ws && plan->ws) {
     hipError_t e = hipFree(plan->ws);
     if (e != hipSuccess) rc = hip_fail(e);
@@ -598,12 +696,11 @@ int ringattn_fwd(ringattn_plan* plan, const void* q, const void* k, const void* 
   if (!q || !k || !v || !out || !lse) return RINGATTN_ERR_NULL;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || ((uintptr_t)lse & 3u)) return RINGATTN_ERR_ALIGN;
   hipStream_t stream = (hipStream_t)stream_;
-  // pair table, merge stream and events: created at the first forward, outside any capture
-  int rc0 = ensure_streams(plan);
+  int rc0 = ensure_tables(plan);
   if (rc0 != RINGATTN_OK) return rc0;
   if (!(plan->p.flags & RINGATTN_FLAG_GRAPH)) return run_forward(plan, q, k, v, out, lse, stream);
 
-  // hipGraph replay: the launches of a forward are captured once per pointer set on a private
+  // hipGraph replay: the launch of a forward is captured once per pointer set on a private
   // stream (kernel nodes only, no memset nodes) and replayed on the caller's stream.
   if (!plan->exec || plan->gq != q || plan->gk != k || plan->gv != v || plan->gout != out || plan->glse != lse) {
     drop_graph(plan);
@@ -639,10 +736,16 @@ int ringattn_block_fwd(ringattn_plan* plan, int step, const void* q, const void*
   if (!q || !k || !v || !o_part || !lse_part) return RINGATTN_ERR_NULL;
   if (step < 0 || step >= plan->p.npes) return RINGATTN_ERR_RANK;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o_part) || ((uintptr_t)lse_part & 3u)) return RINGATTN_ERR_ALIGN;
-  int rc = ensure_streams(plan);
+  int rc = ensure_tables(plan);
   if (rc != RINGATTN_OK) return rc;
-  return launch_items(plan, plan->step_begin[step], plan->step_begin[step + 1] - plan->step_begin[step], q, k, v,
-                      o_part, lse_part, step, (hipStream_t)stream);
+  ringattn::BlockArgs a;
+  fill_geometry(a, plan->p, plan->d);
+  a.q = q;
+  a.k = k;
+  a.v = v;
+  a.o_part = o_part;
+  a.lse_part = lse_part;
+  return launch_slice(plan, plan->step[(size_t)step], a, (hipStream_t)stream);
 }
 
 int ringattn_merge_ring(ringattn_plan* plan, const void* o_parts, const float* lse_parts, void* out,
@@ -650,11 +753,11 @@ int ringattn_merge_ring(ringattn_plan* plan, const void* o_parts, const float* l
   if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
   if (!o_parts || !lse_parts || !out || !lse) return RINGATTN_ERR_NULL;
   if (!aligned16(o_parts) || !aligned16(out) || ((uintptr_t)lse_parts & 3u) || ((uintptr_t)lse & 3u)) return RINGATTN_ERR_ALIGN;
-  for (size_t i = (size_t)plan->all_regions; i < plan->regions.size(); ++i) {
-    int rc = launch_region_merge(plan, o_parts, lse_parts, out, lse, (hipStream_t)stream, plan->regions[i]);
-    if (rc != RINGATTN_OK) return rc;
-  }
-  return RINGATTN_OK;
+  int rc = ensure_tables(plan);
+  if (rc != RINGATTN_OK) return rc;
+  // ONE launch: a grid row per region
+  return launch_regions(plan, 0, plan->n_regions, plan->region_max_len, (int)plan->d.S, plan->d.rows, o_parts, lse_parts,
+                        out, lse, (hipStream_t)stream);
 }
 
 int ringattn_rank_step_fwd(ringattn_plan* plan, int rank, int step, const void* q, const void* k_chunk,
@@ -664,29 +767,23 @@ int ringattn_rank_step_fwd(ringattn_plan* plan, int rank, int step, const void* 
   const int P = plan->p.npes;
   if (rank < 0 || rank >= P || step < 0 || step >= P) return RINGATTN_ERR_RANK;
   if (!aligned16(q) || !aligned16(k_chunk) || !aligned16(v_chunk) || !aligned16(o_part) || ((uintptr_t)lse_part & 3u)) return RINGATTN_ERR_ALIGN;
-  int rc = ensure_streams(plan);
+  int rc = ensure_tables(plan);
   if (rc != RINGATTN_OK) return rc;
-  const int begin = plan->local_begin[rank * P + step], count = plan->local_begin[rank * P + step + 1] - begin;
-  if (count == 0) return RINGATTN_OK;  // nothing of the visited chunk is visible to this rank
   const Derived& d = plan->d;
   const int j = (rank + step) % P;
   const int64_t q_rows = d.start[rank + 1] - d.start[rank], kv_rows = d.start[j + 1] - d.start[j];
-  ringattn::BlockStepArgs a;
+  ringattn::BlockArgs a;
   fill_geometry(a, plan->p, d);
   a.q = q;
   a.k = k_chunk;
   a.v = v_chunk;
   a.o_part = o_part;
   a.lse_part = lse_part;
-  a.items = plan->d_items + begin;
-  a.n_items = count;
   a.bh_stride = q_rows * plan->p.dim;      // every tensor holds one rank's rows only
   a.kv_bh_stride = kv_rows * plan->p.dim;
   a.S = (int)q_rows;
-  a.part_stride_rows = d.BH * q_rows;
-  a.q_tiles_max = (int)((q_rows + ringattn::kBlockM - 1) / ringattn::kBlockM);
-  RA_HIP(ringattn::launch_block_step(a, plan->p.dtype, plan->p.dim, (hipStream_t)stream));
-  return RINGATTN_OK;
+  // an empty slice: nothing of the visited chunk is visible to this rank
+  return launch_slice(plan, plan->local[(size_t)rank * P + step], a, (hipStream_t)stream);
 }
 
 int ringattn_rank_merge(ringattn_plan* plan, int rank, const void* o_parts, const float* lse_parts, void* out,
@@ -695,37 +792,31 @@ int ringattn_rank_merge(ringattn_plan* plan, int rank, const void* o_parts, cons
   if (!o_parts || !lse_parts || !out || !lse) return RINGATTN_ERR_NULL;
   if (rank < 0 || rank >= plan->p.npes) return RINGATTN_ERR_RANK;
   if (!aligned16(o_parts) || !aligned16(out) || ((uintptr_t)lse_parts & 3u) || ((uintptr_t)lse & 3u)) return RINGATTN_ERR_ALIGN;
+  int rc = ensure_tables(plan);
+  if (rc != RINGATTN_OK) return rc;
   const Derived& d = plan->d;
-  const int r0 = d.start[rank], r1 = d.start[rank + 1];
-  for (size_t i = (size_t)plan->all_regions; i < plan->regions.size(); ++i) {
-    const MergeRegion& reg = plan->regions[i];
-    if (reg.start < r0 || reg.start >= r1) continue;
-    ringattn::MergeArgs m;
-    m.o_parts = o_parts;
-    m.lse_parts = lse_parts;
-    m.out = out;
-    m.lse = lse;
-    m.sel_start = reg.start - r0;
-    m.sel_len = reg.len;
-    m.rows = d.BH * reg.len;
-    m.S = r1 - r0;
-    m.part_stride_rows = d.BH * (int64_t)(r1 - r0);
-    m.active = reg.active;
-    m.half_partials = half_partials(plan->p) ? 1 : 0;
-    RA_HIP(ringattn::launch_merge(m, plan->p.dtype, plan->p.dim, (hipStream_t)stream));
-  }
-  return RINGATTN_OK;
+  const int rows = d.start[rank + 1] - d.start[rank];
+  int first = -1, count = 0, max_len = 0;  // the regions of a rank are consecutive
+  for (int i = 0; i < plan->n_regions; ++i)
+    if (plan->region_rank[(size_t)i] == rank) {
+      if (first < 0) first = i;
+      ++count;
+      max_len = std::max(max_len, plan->regions[(size_t)i].len);
+    }
+  if (count == 0) return RINGATTN_OK;
+  return launch_regions(plan, plan->n_regions + first, count, max_len, rows, d.BH * (int64_t)rows, o_parts, lse_parts,
+                        out, lse, (hipStream_t)stream);
 }
 
 int ringattn_plan_work_items(const ringattn_plan* plan, int step, ringattn_work_item* out, int capacity, int* n_out) {
   if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
   if (!n_out || (capacity > 0 && !out)) return RINGATTN_ERR_NULL;
   if (step < -1 || step >= plan->p.npes) return RINGATTN_ERR_RANK;
-  const int begin = step < 0 ? 0 : plan->step_begin[step];
-  const int end = step < 0 ? plan->step_begin[0] : plan->step_begin[step + 1];
+  const int begin = step < 0 ? 0 : plan->step_begin[(size_t)step];
+  const int end = step < 0 ? plan->fwd_items : plan->step_begin[(size_t)step + 1];
   *n_out = end - begin;
   for (int i = begin; i < end && i - begin < capacity; ++i) {
-    const ringattn::WorkItem& w = plan->h_items[i];
+    const ringattn::WorkItem& w = plan->h_items[(size_t)i];
     out[i - begin] = ringattn_work_item{w.q_start, w.q_len, w.kv_start, w.kv_len, w.diag_off, w.slot};
   }
   return RINGATTN_OK;
@@ -735,11 +826,10 @@ int ringattn_plan_launch_times(ringattn_plan* plan, float* ms, int capacity, int
   if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
   if (!n_out || (capacity > 0 && !ms)) return RINGATTN_ERR_NULL;
   if (!plan->timed_forward) return RINGATTN_ERR_PLAN;
-  const int n = (int)plan->groups.size();
-  *n_out = n;
-  for (int g = 0; g < n && g < capacity; ++g) {
-    RA_HIP(hipEventSynchronize(plan->ev_t1[g]));
-    RA_HIP(hipEventElapsedTime(&ms[g], plan->ev_t0[g], plan->ev_t1[g]));
+  *n_out = 1;
+  if (capacity > 0) {
+    RA_HIP(hipEventSynchronize(plan->ev_t1));
+    RA_HIP(hipEventElapsedTime(&ms[0], plan->ev_t0, plan->ev_t1));
   }
   return RINGATTN_OK;
 }
@@ -747,10 +837,10 @@ int ringattn_plan_launch_times(ringattn_plan* plan, float* ms, int capacity, int
 int ringattn_plan_merge_regions(const ringattn_plan* plan, int* start, int* len, uint64_t* active, int capacity, int* n_out) {
   if (!plan_ok(plan)) return RINGATTN_ERR_PLAN;
   if (!n_out || (capacity > 0 && (!start || !len || !active))) return RINGATTN_ERR_NULL;
-  const int n = (int)plan->regions.size() - plan->all_regions;
+  const int n = plan->n_regions;
   *n_out = n;
   for (int i = 0; i < n && i < capacity; ++i) {
-    const MergeRegion& m = plan->regions[plan->all_regions + i];
+    const ringattn::MergeRegion& m = plan->regions[(size_t)i];
     start[i] = m.start;
     len[i] = m.len;
     active[i] = m.active;
@@ -766,19 +856,24 @@ int ringattn_merge(const float* o_parts, const float* lse_parts, int n_parts, in
   if (dtype != RINGATTN_DTYPE_FP16 && dtype != RINGATTN_DTYPE_BF16) return RINGATTN_ERR_DTYPE;
   if (rows < 0 || rows > ((int64_t)1 << 40)) return RINGATTN_ERR_SHAPE;
   if (!aligned16(o_parts) || !aligned16(out)) return RINGATTN_ERR_ALIGN;
-  ringattn::MergeArgs m;
-  m.o_parts = o_parts;
-  m.lse_parts = lse_parts;
-  m.out = out;
-  m.lse = lse;
-  m.rows = rows;
-  m.part_stride_rows = rows;
-  m.active = n_parts >= 64 ? ~(uint64_t)0 : (((uint64_t)1 << n_parts) - 1);
-  m.half_partials = 0;
-  m.S = (int)(rows > 0 ? (rows < INT32_MAX ? rows : INT32_MAX) : 1);
-  m.sel_start = 0;
-  m.sel_len = m.S;
-  RA_HIP(ringattn::launch_merge(m, dtype, dim, (hipStream_t)stream));
+  // one launch per 2^30 rows (a launch's row count is an int)
+  const int64_t kChunk = (int64_t)1 << 30;
+  for (int64_t r0 = 0; r0 < rows; r0 += kChunk) {
+    const int len = (int)std::min(kChunk, rows - r0);
+    ringattn::MergeArgs m;
+    std::memset(&m, 0, sizeof(m));
+    m.o_parts = o_parts + r0 * dim;
+    m.lse_parts = lse_parts + r0;
+    m.out = (char*)out + r0 * dim * 2;
+    m.lse = lse + r0;
+    m.single = ringattn::MergeRegion{0, len, n_parts >= 64 ? ~(uint64_t)0 : (((uint64_t)1 << n_parts) - 1)};
+    m.n_regions = 1;
+    m.max_len = len;
+    m.heads = 1;
+    m.S = len;
+    m.part_stride_rows = rows;
+    RA_HIP(ringattn::launch_merge(m, dtype, dim, (hipStream_t)stream));
+  }
   return RINGATTN_OK;
 }
 

@@ -9,12 +9,13 @@ namespace ringattn {
 constexpr int kBlockM = 128;  // query rows per workgroup (4 waves x 32 rows)
 constexpr int kMaxParts = 64; // partial slots a merge can combine
 
-// One unit of block-attention work: the queries [q_start, q_start + q_len) of every head
-// against the keys/values [kv_start, kv_start + kv_len) of the matching KV head -- the body
-// of one ring step of one rank (csrc/ring_attention.cu:456-470,531-610: rank r at step s
-// works on the KV chunk of rank (r + s) mod P).  Row numbers are local to a head's [S, D]
-// slab and need not be multiples of any tile size.  The normalised partial O and the partial LSE
-// of the item go to partial slot `slot`, at the rows of its queries.
+// One unit of block-attention work as the host layer lists it: the queries
+// [q_start, q_start + q_len) of every head against the keys/values
+// [kv_start, kv_start + kv_len) of the matching KV head -- the body of one ring step of one
+// rank (csrc/ring_attention.cu:456-470,531-610: rank r at step s works on the KV chunk of rank
+// (r + s) mod P).  Row numbers are local to a head's [S, D] slab and need not be multiples of
+// any tile size.  The normalised partial O and the partial LSE of the item go to partial slot
+// `slot`, at the rows of its queries.
 struct WorkItem {
   int q_start, q_len;
   int kv_start, kv_len;
@@ -24,54 +25,94 @@ struct WorkItem {
   int slot;
   int pad0, pad1;
 };
-static_assert(sizeof(WorkItem) == 32, "WorkItem is read as two 16-byte scalar loads");
 
-struct BlockStepArgs {
+// What the block kernel runs: a SEGMENT is a range of query rows (of every head) together with
+// ALL the key ranges it meets -- the ring steps of the reference's step loop
+// (csrc/ring_attention.cu:456-620) for those rows.  One workgroup owns 128 rows of a segment,
+// keeps their Q in registers and walks the segment's items, as the reference's CTA walks the
+// ring steps (:439-443,456), emitting one (partial O, partial LSE) per item.
+struct SegItem {
+  int kv_start, kv_len;
+  int diag_off;         // as in WorkItem, relative to the first row of the segment
+  int part_bh_stride;   // rows between consecutive heads in this item's partial block
+  int64_t part_base;    // row (in the partial buffers) of the segment's first row of head 0
+  int slot;             // ring step, for inspection only
+  int pad;
+};
+static_assert(sizeof(SegItem) == 32, "SegItem is read as two 16-byte scalar loads");
+
+struct Segment {
+  int q_start, q_len;
+  int item_begin, item_count;  // slice of the SegItem table, in ascending ring-step order
+  int last_item;               // index (within the slice) of the item to run last, -1: table order.
+                               // A masked (diagonal) item runs last: its length differs per q tile,
+                               // and the q tiles that share a KV chunk in L2 stay in step until then.
+  int reverse_tiles;           // the q tiles with the most visible keys are scheduled first
+  int pad0, pad1;
+};
+static_assert(sizeof(Segment) == 32, "Segment is read as two 16-byte scalar loads");
+
+struct BlockArgs {
   const void* q;       // [BH, S, D] storage dtype
   const void* k;       // [batch * heads / kv_group, S, D]
   const void* v;       // [batch * heads / kv_group, S, D]
-  void* o_part;        // partial slot `slot_bias`: [BH, S, D] partial O (normalised), fp32 or fp16 (half_partials)
-  float* lse_part;     // partial slot `slot_bias`: [BH, S] fp32 partial LSE (natural log)
-  const WorkItem* items;     // device array
-  int64_t bh_stride;   // elements between heads of q (= S * D)
+  void* o_part;        // partial O rows (normalised), fp32 or fp16 (half_partials); indexed by SegItem::part_base
+  float* lse_part;     // partial LSE rows (natural log), same row numbering
+  void* out;           // fuse_merge: [BH, S, D] storage dtype
+  float* lse;          // fuse_merge: [BH, S]
+  const Segment* segs; // device arrays
+  const SegItem* items;
+  const int2* groups;  // NULL, or [8][groups_per_xcd] (segment, head) pairs: what the workgroups of each XCD run,
+                       // in order; segment < 0 marks an unused entry
+  int groups_per_xcd;
+  int64_t bh_stride;   // elements between heads of q and out (= S * D)
   int64_t kv_bh_stride;      // elements between heads of k and v
-  int64_t part_stride_rows;  // rows between consecutive partial slots
-  int S;               // rows per head in the partial slots
-  int q_tiles_max;     // kBlockM-row q tiles of the longest item (grid dimension)
-  int n_items;
-  int slot_bias;       // item.slot - slot_bias is the slot index relative to o_part / lse_part
+  int S;               // rows per head of q, out and lse
+  int q_tiles_max;     // kBlockM-row q tiles of the longest segment (grid dimension)
+  int n_segs;
   int BH;              // batch * heads
   int heads;           // query heads per batch entry
   int kv_group;        // query heads per KV head (1 = one KV head per query head)
   float scale_log2;    // softmax_scale * log2(e)
   int half_partials;   // partial O stored as fp16 instead of fp32
+  int fuse_merge;      // after its last item a workgroup merges the partials of its rows into out / lse
 };
 
-// Merge of (O, LSE) partials into the final O (storage dtype) and LSE, for the rows
-// [sel_start, sel_start + sel_len) of every head.
+// Merge of (O, LSE) partials into the final O (storage dtype) and LSE, for row ranges of every
+// head: a region covers rows [start, start + len) and reads the slots whose bit is set in `active`.
+struct MergeRegion {
+  int start, len;
+  uint64_t active;
+};
+static_assert(sizeof(MergeRegion) == 16, "MergeRegion is read as one 16-byte scalar load");
+
 struct MergeArgs {
   const void* o_parts;    // [slots, heads * S, D] fp32, or fp16 with half_partials
   const float* lse_parts; // [slots, heads * S]
   void* out;              // [heads * S, D] storage dtype
   float* lse;             // [heads * S]
-  int64_t rows;           // heads * sel_len rows are merged
-  int64_t part_stride_rows;  // rows between consecutive slots (>= heads * S)
-  uint64_t active;        // bit s set: slot s holds a partial for these rows; other slots are never read
+  const MergeRegion* regions;  // device array of n_regions entries, one grid row each; NULL: `single`
+  MergeRegion single;
+  int n_regions;          // 1 with `single`
+  int max_len;            // longest region (grid columns)
+  int heads;              // batch * heads: every region is merged for each of them
   int S;                  // rows per head
-  int sel_start, sel_len; // row range within a head
+  int64_t part_stride_rows;  // rows between consecutive slots (>= heads * S)
   int half_partials;
 };
 
-// Up to kMaxParts work items passed BY VALUE to a small kernel that writes them to device
+// Up to kMaxParts table entries passed BY VALUE to a small kernel that writes them to device
 // memory: an item table for callers that may not copy from the host (no allocation, no
 // memcpy node: a plain kernel launch).
-struct ItemPack {
-  WorkItem items[kMaxParts];
+struct TablePack {
+  Segment seg;
+  SegItem items[kMaxParts];
 };
 
 // dtype: 0 = fp16, 1 = bf16.  Return hipSuccess or the launch error.
-hipError_t launch_block_step(const BlockStepArgs& a, int dtype, int dim, hipStream_t stream);
+hipError_t launch_block(const BlockArgs& a, int dtype, int dim, hipStream_t stream);
 hipError_t launch_merge(const MergeArgs& a, int dtype, int dim, hipStream_t stream);
-hipError_t launch_write_items(const ItemPack& pack, int n, WorkItem* dst, hipStream_t stream);
+// writes pack.seg to *seg_dst and pack.items[0..n) to item_dst
+hipError_t launch_write_table(const TablePack& pack, int n, Segment* seg_dst, SegItem* item_dst, hipStream_t stream);
 
 }  // namespace ringattn

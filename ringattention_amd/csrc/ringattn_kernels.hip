@@ -1,8 +1,11 @@
 // gfx950 (CDNA4) kernels for the ring-attention forward path.
 //
-//   block_attention_kernel : one ring step for every active virtual rank --
+//   block_attention_kernel : the ring steps of every virtual rank.  A workgroup owns 128
+//       query rows, keeps their Q in registers and walks the KV chunks those rows meet (the
+//       reference's CTA loops over the ring steps in the same way, csrc/ring_attention.cu:
+//       439-443,456), per chunk
 //       S^T = K Q^T, online softmax with running max / sum, O^T += V^T P^T,
-//       emitting a normalised fp32 partial O and a natural-log fp32 LSE.
+//       emitting a normalised fp32 partial O and a natural-log fp32 LSE per chunk.
 //       It restates the inner KV-tile loop of the reference kernel
 //       (csrc/ring_attention.cu:536-610: gemm_smem :278-301, softmax_rescale_o
 //       :194-245 completed with the missing `sum += sum_cur` tail,
@@ -32,6 +35,7 @@
 #include "ringattn_kernels.h"
 
 #include <type_traits>
+
 
 namespace ringattn {
 
@@ -106,8 +110,120 @@ template <int D> static __device__ __forceinline__ int v_swizzle(int row) {
                   : ((((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1));
 }
 
-// ---- block attention: one ring step for every active virtual rank ------------------------
-// The KV chunk is consumed in 32-key tiles held in two 4-deep LDS rings (K and V), filled by
+// ---- merge of one row: shared by the merge kernel and the block kernel's fused merge -------
+template <int DT> struct Store8;
+template <> struct Store8<0> {
+  static __device__ __forceinline__ void st(void* p, const float* x) {
+    f16x8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (_Float16)x[e];
+    *(f16x8*)p = v;
+  }
+};
+template <> struct Store8<1> {
+  static __device__ __forceinline__ void st(void* p, const float* x) {
+    bf16x8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (__bf16)x[e];
+    *(bf16x8*)p = v;
+  }
+};
+
+// 8 consecutive columns of one partial row as floats
+template <bool HP> struct PartRow;
+template <> struct PartRow<false> {
+  using ptr = const float*;
+  static __device__ __forceinline__ void ld(ptr p, f32x4& x0, f32x4& x1) {
+    x0 = *(const f32x4*)p;
+    x1 = *(const f32x4*)(p + 4);
+  }
+};
+template <> struct PartRow<true> {
+  using ptr = const _Float16*;
+  static __device__ __forceinline__ void ld(ptr p, f32x4& x0, f32x4& x1) {
+    const f16x8 v = *(const f16x8*)p;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      x0[e] = (float)v[e];
+      x1[e] = (float)v[4 + e];
+    }
+  }
+};
+
+// The parts of one row, in ascending slot order: the set bits of a mask over equally spaced slots.
+struct SlotParts {
+  uint64_t rest;
+  int64_t row, stride;  // the row in slot 0, rows between slots
+  __device__ __forceinline__ int left() const { return __builtin_popcountll(rest); }
+  __device__ __forceinline__ int64_t take() {
+    const int64_t r = row + (int64_t)__builtin_ctzll(rest) * stride;
+    rest &= rest - 1;
+    return r;
+  }
+};
+// L = logsumexp_s L_s, O = sum_s exp(L_s - L) O_s over the parts of one row; this thread owns
+// columns [8 c8, 8 c8 + 8).  A part with L_s = -inf is the identity and its O is not used.
+template <int DT, int D, bool HP, class Parts>
+static __device__ __forceinline__ void merge_row(Parts parts, const void* o_parts, const float* lse_parts,
+                                                 void* out, float* lse, int64_t out_row, int c8) {
+  const typename PartRow<HP>::ptr o_base = (typename PartRow<HP>::ptr)o_parts + c8 * 8;
+  float mx = -INFINITY;
+  {
+    Parts p = parts;
+    while (p.left()) mx = fmaxf(mx, lse_parts[p.take()]);
+  }
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  float wsum = 0.f;
+  if (mx != -INFINITY) {
+    // four parts per iteration: all their loads are issued before the first is consumed
+    Parts p = parts;
+    while (p.left() >= 4) {
+      float L[4];
+      f32x4 x0[4], x1[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t r = p.take();
+        L[u] = lse_parts[r];
+        PartRow<HP>::ld(o_base + r * D, x0[u], x1[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float w = __expf(L[u] - mx);
+        if (L[u] == -INFINITY) continue;  // identity element: its O may hold anything
+        wsum += w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          acc[e] = __builtin_fmaf(w, x0[u][e], acc[e]);
+          acc[4 + e] = __builtin_fmaf(w, x1[u][e], acc[4 + e]);
+        }
+      }
+    }
+    while (p.left()) {
+      const int64_t r = p.take();
+      const float Ls = lse_parts[r];
+      const float w = __expf(Ls - mx);
+      f32x4 x0, x1;
+      PartRow<HP>::ld(o_base + r * D, x0, x1);
+      if (Ls == -INFINITY) continue;
+      wsum += w;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[e] = __builtin_fmaf(w, x0[e], acc[e]);
+        acc[4 + e] = __builtin_fmaf(w, x1[e], acc[4 + e]);
+      }
+    }
+    const float inv = 1.f / wsum;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] *= inv;
+  }
+  Store8<DT>::st((char*)out + (out_row * D + c8 * 8) * 2, acc);
+  if (c8 == 0) lse[out_row] = (mx == -INFINITY) ? -INFINITY : mx + __logf(wsum);
+}
+
+// ---- block attention: the ring steps of 128 query rows ----------------------------------
+// A KV chunk is consumed in 32-key tiles held in two 4-deep LDS rings (K and V), filled by
 // direct-to-LDS loads that run two blocks ahead.  Block u of the loop runs, in ONE
 // instruction stream,
 //     MFMAs of S^T(u+1) = K(u+1) Q^T      next to   the exponentials of tile u,
@@ -119,8 +235,11 @@ template <int D> static __device__ __forceinline__ int v_swizzle(int row) {
 // branches.  Until then p = exp2((s - m) k2) may exceed 1 (by at most 2^kLazyLog2, well
 // inside fp16 and bf16 range); O = acc / l and LSE = (m k2 + log2 l) ln 2 do not depend on
 // the choice of m.
+// From one KV chunk to the next the tile pipeline keeps running where the shapes allow it
+// (the loads that run ahead of the last tiles fetch the first tiles of the next chunk); the
+// softmax state is emitted as that chunk's partial and reset.
 template <int DT, int D, bool HP>
-__global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStepArgs a) {
+__global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockArgs a) {
   using E = Elem<DT>;
   constexpr int QB = 1;            // 32-query blocks per wave
   constexpr int BM = kBlockM;      // query rows per workgroup: 4 waves x 32
@@ -140,45 +259,45 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 31, h = lane >> 5;
 
-  // workgroup -> (head, work item, q tile).  blockIdx mod 8 is the XCD: the q tiles of a
-  // (head, item) group stay on one XCD and share its K and V in that L2.  Groups are
-  // head-major (the items of a head run together) over an ODD item count (the host pads by
-  // one empty item if needed): an XCD takes every 8th group and so cycles through all items;
-  // with a count sharing a factor with 8 it would get the same few items for every head,
-  // and items differ in cost.
+  // workgroup -> (segment, head, q tile).  blockIdx mod 8 is the XCD: the q tiles of a
+  // (segment, head) group stay on one XCD and share its K and V in that L2.  Groups are
+  // segment-major and the host lists the segments by decreasing work, so the workgroups that
+  // are dispatched last are the short ones.
+  // With a group table the host has dealt the heads to the XCDs and listed, per XCD, the
+  // segments of one head after the other: ranks of a head follow each other through the same
+  // K and V, which then stay in that XCD's L2 / the memory-side cache.
   const int q_tiles = a.q_tiles_max;
-  const int n_pad = a.n_items | 1;
-  const int groups = n_pad * a.BH;
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int group = (slot / q_tiles) * 8 + xcd;
-  if (group >= groups) return;
-  const int bh = group / n_pad, item = group % n_pad;
-  if (item >= a.n_items) return;
-  const WorkItem w = a.items[item];
-  const bool diag = w.diag_off >= 0;
-  const int q_start = w.q_start, q_len = w.q_len;
-  const int kv_start = w.kv_start, kv_len = w.kv_len;
-  int qt = slot % q_tiles;
-  if (qt * BM >= q_len) return;  // items shorter than the longest one
-  if (diag) qt = (q_len + BM - 1) / BM - 1 - qt;  // most keys first
-  const int diag_rows = w.diag_off + qt * BM;  // keys below this local index are visible to the whole q tile
-  // Lengths need not be multiples of the tile sizes (the predication the reference leaves as
-  // a TODO, csrc/ring_attention.cu:143-145).  The last key tile may reach beyond the KV range:
-  // its loads are clamped to the last valid row and its surplus keys masked.  Query rows
-  // beyond the range are computed on a copy of the last valid row and not stored.
-  const int kv_tiles = (kv_len + BN - 1) / BN;
-  const int kv_tail = (kv_len % BN) ? kv_len / BN : -1;  // the tile with surplus keys, if any
-  const int n_tiles = diag ? min(kv_tiles, (diag_rows + BM + BN - 1) / BN) : kv_tiles;
-  // tiles >= first_masked need a mask (causal diagonal or surplus keys)
-  const int first_masked = min(diag ? diag_rows / BN : n_tiles, kv_tail >= 0 ? kv_tail : n_tiles);
+  const int xcd = blockIdx.x & 7, wslot = blockIdx.x >> 3;
+  int sg, bh;
+  if (a.groups) {
+    const int2 g = a.groups[xcd * a.groups_per_xcd + wslot / q_tiles];
+    sg = g.x;
+    bh = g.y;
+    if (sg < 0) return;
+  } else {
+    const int group = (wslot / q_tiles) * 8 + xcd;
+    if (group >= a.n_segs * a.BH) return;
+    sg = group / a.BH;
+    bh = group % a.BH;
+  }
+  const Segment seg = a.segs[sg];
+  const int q_start = seg.q_start, q_len = seg.q_len;
+  int qt = wslot % q_tiles;
+  if (qt * BM >= q_len) return;  // segments shorter than the longest one
+  if (seg.reverse_tiles) qt = (q_len + BM - 1) / BM - 1 - qt;  // most keys first
+  const int n_items = seg.item_count;
+  // items in run order: table order, except that item `last_item` is moved to the end
+  auto item_at = [&](int i) -> const SegItem* {
+    int idx = i;
+    if (seg.last_item >= 0) idx = (i == n_items - 1) ? seg.last_item : (i >= seg.last_item ? i + 1 : i);
+    return a.items + seg.item_begin + idx;
+  };
 
   const int64_t head_off = (int64_t)bh * a.bh_stride;
   // grouped-query attention: query head h of a batch entry reads KV head h / kv_group
   const int kv_bh = (bh / a.heads) * (a.heads / a.kv_group) + (bh % a.heads) / a.kv_group;
   const int64_t kv_head_off = (int64_t)kv_bh * a.kv_bh_stride;
   const char* qbase = (const char*)a.q + (head_off + (int64_t)(q_start + qt * BM) * D) * 2;
-  const char* kbase = (const char*)a.k + (kv_head_off + (int64_t)kv_start * D) * 2;
-  const char* vbase = (const char*)a.v + (kv_head_off + (int64_t)kv_start * D) * 2;
 
   // this lane's query rows (local to the q tile): 32 QB wave + 32 qb + n
   s16x8 qf[QB][KS];
@@ -215,31 +334,66 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
   float ms[QB];  // m * k2, 0 while m is -inf (guard of csrc/ring_attention.cu:183)
   float ls[QB][4];
   f32x16 oacc[QB][DB];
+  auto reset_state = [&]() {
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    m[qb] = -INFINITY;
-    ms[qb] = 0.f;
+    for (int qb = 0; qb < QB; ++qb) {
+      m[qb] = -INFINITY;
+      ms[qb] = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) ls[qb][i] = 0.f;
+      for (int i = 0; i < 4; ++i) ls[qb][i] = 0.f;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+      for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) oacc[qb][db][e] = 0.f;
-  }
+        for (int e = 0; e < 16; ++e) oacc[qb][db][e] = 0.f;
+    }
+  };
+  reset_state();
   f32x16 s_even[QB], s_odd[QB];
   s16x8 pf[QB][2];
+
+  // ---- the KV chunk being walked (wave-uniform)
+  const char *kbase = nullptr, *vbase = nullptr;
+  // where the loads that run past the last tile go: the first tiles of the next chunk when
+  // the pipeline carries over (stride TILE), else a re-read of the last tile (stride 0)
+  int64_t kpast_delta = 0, vpast_delta = 0;  // from the end of this chunk's K (V) to that place
+  int past_stride = 0;
+  int kv_len = 0, n_tiles = 0, first_masked = 0, kv_tail = -1, diag_rows = 0;
+  bool diag = false;
+  // Lengths need not be multiples of the tile sizes (the predication the reference leaves as
+  // a TODO, csrc/ring_attention.cu:143-145).  The last key tile may reach beyond the KV range:
+  // its loads are clamped to the last valid row and its surplus keys masked.  Query rows
+  // beyond the range are computed on a copy of the last valid row and not stored.
+  auto set_chunk = [&](const SegItem* w) {
+    diag = w->diag_off >= 0;
+    kv_len = w->kv_len;
+    diag_rows = w->diag_off + qt * BM;  // keys below this local index are visible to the whole q tile
+    const int kv_tiles = (kv_len + BN - 1) / BN;
+    kv_tail = (kv_len % BN) ? kv_len / BN : -1;  // the tile with surplus keys, if any
+    n_tiles = diag ? min(kv_tiles, (diag_rows + BM + BN - 1) / BN) : kv_tiles;
+    // tiles >= first_masked need a mask (causal diagonal or surplus keys)
+    first_masked = min(diag ? diag_rows / BN : n_tiles, kv_tail >= 0 ? kv_tail : n_tiles);
+    kbase = (const char*)a.k + (kv_head_off + (int64_t)w->kv_start * D) * 2;
+    vbase = (const char*)a.v + (kv_head_off + (int64_t)w->kv_start * D) * 2;
+  };
 
   // bytes to step back so that a row of tile kv_tail beyond the KV range reads the last valid row
   auto surplus = [&](int i) {
     const int row = ((wave * LD + i) * 64 + lane) / CPR;
     return max(0, kv_tail * BN + row - (kv_len - 1)) * ROWB;
   };
-  // `checked`: the tile may be kv_tail (steady blocks never issue that one)
-  // A tile index at or beyond n_tiles names a PHANTOM tile: steady blocks run to the end of
-  // the loop and keep loading two blocks ahead; such a load re-reads the last tile into the
-  // ring slot the phantom would use, which no block reads any more.
+  // Byte offset of tile t from the chunk's first tile, in branch-free scalar arithmetic (a
+  // branch would split the steady blocks): t < n_tiles gives t TILE; beyond that
+  // n_tiles TILE + delta + (t - n_tiles) past_stride, delta being the distance from the end of
+  // this chunk to where such loads go.
+  auto tile_offset = [&](int t, int64_t delta) -> int64_t {
+    const int64_t beyond = (int64_t)((n_tiles - 1 - t) >> 31);  // all ones iff t >= n_tiles
+    return (int64_t)min(t, n_tiles) * TILE + (int64_t)max(t - n_tiles, 0) * past_stride + (delta & beyond);
+  };
+  // `checked`: the tile may be kv_tail (steady blocks never issue that one); checked calls
+  // name existing tiles only.  A tile index at or beyond n_tiles comes from a steady block
+  // that keeps loading two blocks ahead at the end of the chunk.
   auto issue_k = [&](int t, auto checked) {
-    const char* kt = kbase + (int64_t)min(t, n_tiles - 1) * TILE;
+    const char* kt = kbase + tile_offset(t, kpast_delta);
     const unsigned kd = __builtin_amdgcn_readfirstlane(smem_base + (t & (NBUF - 1)) * TILE + wave * (LD * 1024));
     if (decltype(checked)::value && t == kv_tail) {
 #pragma unroll
@@ -250,7 +404,7 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
     }
   };
   auto issue_v = [&](int t, auto checked) {
-    const char* vt = vbase + (int64_t)min(t, n_tiles - 1) * TILE;
+    const char* vt = vbase + tile_offset(t, vpast_delta);
     const unsigned vd = __builtin_amdgcn_readfirstlane(smem_base + (NBUF + (t & (NBUF - 1))) * TILE + wave * (LD * 1024));
     if (decltype(checked)::value && t == kv_tail) {
 #pragma unroll
@@ -304,12 +458,14 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
     return cross_half_max(fmaxf(m0, m1));
   };
   // cand = max(m, tile max).  The reference moves when some row's cand is far above it (or it
-  // is still unset): rescale of l and acc-O as in csrc/ring_attention.cu:226-232.
-  auto move_reference = [&](const float (&cand)[QB]) {
+  // is still unset): rescale of l and acc-O as in csrc/ring_attention.cu:226-232.  `live` is
+  // false for the scores a steady block computes beyond the last tile of a chunk: they belong
+  // to the next chunk (or to nothing) and must not touch this chunk's state.
+  auto move_reference = [&](const float (&cand)[QB], bool live) {
     bool far = false;
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) far = far || ((cand[qb] - m[qb]) * a.scale_log2 > kLazyLog2);
-    if (__builtin_amdgcn_ballot_w64(far) != 0) {
+    if (live && __builtin_amdgcn_ballot_w64(far) != 0) {
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         const float cs = (cand[qb] == -INFINITY) ? 0.f : cand[qb] * a.scale_log2;
@@ -321,6 +477,14 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
         m[qb] = cand[qb];
         ms[qb] = cs;
       }
+    }
+  };
+  // the first tile of a chunk sets the reference: l and acc-O are zero, nothing to rescale
+  auto set_reference = [&](const float (&cand)[QB]) {
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      m[qb] = cand[qb];
+      ms[qb] = (cand[qb] == -INFINITY) ? 0.f : cand[qb] * a.scale_log2;
     }
   };
   // P^T = exp2(S^T k2 - m k2): row sum from the unrounded values (csrc/ring_attention.cu:242),
@@ -362,11 +526,15 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
     for (int qb = 0; qb < QB; ++qb) cand[qb] = tile_max(sacc[qb], m[qb]);
   };
 
+  // Set between a carried-over chunk boundary and the first pair of the next chunk: the tiles
+  // that pair needs were waited for (and the barrier passed) BEFORE the partial was stored, so
+  // that the pair does not wait for those stores (stores count in vmcnt too).
+  bool synced = false;
   // Block u.  Even blocks start with the barrier of the pair (u, u+1): K(u+1), K(u+2), V(u)
   // and V(u+1), issued during the previous pair, have landed, and every wave is past block
   // u-1, so the ring slots of K(u-1), K(u), V(u-2), V(u-1) are free for K(u+3), K(u+4),
   // V(u+2), V(u+3), which are issued during this pair.
-  // STEADY blocks (all those tiles exist, tiles u+1 and u+2 unmasked) have compile-time ring
+  // STEADY blocks (tiles u+1 and u+2 unmasked or covered by MASKED) have compile-time ring
   // slots and no conditions.
   auto block = [&](auto slot_c, auto steady, auto masked, int u) {
     constexpr int SLOT = decltype(slot_c)::value;  // u mod 4 (STEADY) or u mod 2 (general)
@@ -379,8 +547,12 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
       // the four tile loads of a pair are spread over its two blocks instead of being
       // issued in one burst behind the barrier
       if ((SLOT & 1) == 0) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+        if (SLOT == 0 && synced) {
+          synced = false;  // a carried chunk's first pair: its wait and barrier came before the partial was stored
+        } else {
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          __syncthreads();
+        }
         issue_k(u + 3, kUnchecked);
       } else {
         issue_v(u + 1, kUnchecked);
@@ -400,11 +572,15 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
       }
-      move_reference(cand);
+      move_reference(cand, u + 1 < n_tiles);
     } else {
       if ((u & 1) == 0) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+        if (synced) {
+          synced = false;
+        } else {
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          __syncthreads();
+        }
         if (u + 3 < n_tiles) issue_k(u + 3, kChecked);
         if (u + 4 < n_tiles) issue_k(u + 4, kChecked);
         if (u + 2 < n_tiles) issue_v(u + 2, kChecked);
@@ -418,213 +594,241 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockStep
       pv_product(u & 3);
       if (u + 1 < n_tiles) {
         tile_maxes(nxt, cand);
-        move_reference(cand);
+        move_reference(cand, true);
       }
     }
   };
 
-  // the first tiles go out next to the Q loads: one memory latency for all of them
-  issue_k(0, kChecked);
-  if (n_tiles > 1) issue_k(1, kChecked);
-  if (n_tiles > 2) issue_k(2, kChecked);
-  issue_v(0, kChecked);
-  if (n_tiles > 1) issue_v(1, kChecked);
-  __builtin_amdgcn_s_waitcnt(0);  // retire the Q loads with a wait the compiler can see (and the tiles)
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  {
-    float cand[QB];
-    qk(s_even, 0);
-    mask_tile(s_even, 0, kUnchecked);
-    tile_maxes(s_even, cand);
-    move_reference(cand);
-  }
+  // this chunk's partial (csrc/ring_attention.cu:621-633): normalise, emit O and LSE
+  auto emit_partial = [&](const SegItem* w) {
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      const float l = cross_half_sum((ls[qb][0] + ls[qb][1]) + (ls[qb][2] + ls[qb][3]));
+      const float inv = (l > 0.f) ? 1.f / l : 0.f;
+      const int row_l = qt * BM + 32 * QB * wave + 32 * qb + n;
+      if (row_l >= q_len) continue;  // a row beyond the query range
+      const int64_t prow = w->part_base + (int64_t)bh * w->part_bh_stride + row_l;
+      const int64_t opos = prow * D;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          f32x4 val;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) val[e] = oacc[qb][db][4 * q4 + e] * inv;
+          if (HP) {  // fp16 partials: |O_part| <= max |V|, the caller vouches that this fits
+            f16x4 hv;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) hv[e] = (_Float16)val[e];
+            *(f16x4*)((_Float16*)a.o_part + opos + 32 * db + 8 * q4 + 4 * h) = hv;
+          } else {
+            *(f32x4*)((float*)a.o_part + opos + 32 * db + 8 * q4 + 4 * h) = val;
+          }
+        }
+      if (h == 0) {
+        const float lse = (l > 0.f) ? (ms[qb] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
+        a.lse_part[prow] = lse;
+      }
+    }
+  };
 
   using C0 = std::integral_constant<int, 0>;
   using C1 = std::integral_constant<int, 1>;
   using C2 = std::integral_constant<int, 2>;
   using C3 = std::integral_constant<int, 3>;
-  // Steady blocks come in groups of four (ring slots are compile-time constants).  A group
-  // starting at u computes the scores of tiles u+1 .. u+4 and loads up to tile u+6:
-  //   plain groups   while those four tiles need no mask; without any mask in the item the last
-  //                  group runs up to tile n_tiles-1 and its last block computes (and drops)
-  //                  the scores of a phantom tile;
-  //   masked groups  (diagonal items) for the rest: every block masks its tile u+1;
-  //   an item with surplus keys in its last tile keeps clear of that tile (its loads need the
-  //   clamped form) and leaves the rest to the general blocks.
-  const bool ragged = kv_tail >= 0;
-  const int plain_end = ragged ? min(first_masked, kv_tail - 2) : (diag ? first_masked : n_tiles + 1);
-  const int masked_end = (diag && !ragged) ? n_tiles + 1 : 0;
-  int u = 0;
-  for (; u + 4 < plain_end; u += 4) {
-    block(C0{}, std::true_type{}, std::false_type{}, u);
-    block(C1{}, std::true_type{}, std::false_type{}, u + 1);
-    block(C2{}, std::true_type{}, std::false_type{}, u + 2);
-    block(C3{}, std::true_type{}, std::false_type{}, u + 3);
-  }
-  for (; u + 4 < masked_end; u += 4) {
-    block(C0{}, std::true_type{}, std::true_type{}, u);
-    block(C1{}, std::true_type{}, std::true_type{}, u + 1);
-    block(C2{}, std::true_type{}, std::true_type{}, u + 2);
-    block(C3{}, std::true_type{}, std::true_type{}, u + 3);
-  }
-  for (; u < n_tiles; ++u) {
-    if (u & 1) block(C1{}, std::false_type{}, std::false_type{}, u);
-    else block(C0{}, std::false_type{}, std::false_type{}, u);
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // phantom loads may still be in flight
 
-  // epilogue (csrc/ring_attention.cu:621-633): normalise, emit partial O and LSE
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    const float l = cross_half_sum((ls[qb][0] + ls[qb][1]) + (ls[qb][2] + ls[qb][3]));
-    const float inv = (l > 0.f) ? 1.f / l : 0.f;
-    const int row_l = qt * BM + 32 * QB * wave + 32 * qb + n;
-    if (row_l >= q_len) continue;  // a row beyond the query range
-    const int row_g = q_start + row_l;
-    const int64_t slot_rows = (int64_t)(w.slot - a.slot_bias) * a.part_stride_rows;
-    const int64_t opos = (slot_rows + (int64_t)bh * a.S + row_g) * D;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        f32x4 val;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) val[e] = oacc[qb][db][4 * q4 + e] * inv;
-        if (HP) {  // fp16 partials: |O_part| <= max |V|, the caller vouches that this fits
-          f16x4 hv;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) hv[e] = (_Float16)val[e];
-          *(f16x4*)((_Float16*)a.o_part + opos + 32 * db + 8 * q4 + 4 * h) = hv;
-        } else {
-          *(f32x4*)((float*)a.o_part + opos + 32 * db + 8 * q4 + 4 * h) = val;
-        }
+  bool carried = false;  // the previous chunk's pipeline ran on into this one
+  for (int it = 0; it < n_items; ++it) {
+    const SegItem* w = item_at(it);
+    set_chunk(w);
+    // The pipeline carries over into the next chunk when this one ends in plain steady groups
+    // on a multiple of four tiles (ring slots then line up with a fresh start) and the next
+    // chunk has its first three tiles in full.
+    bool carry = false;
+    if (it + 1 < n_items) {
+      const SegItem* wn = item_at(it + 1);
+      carry = !diag && kv_tail < 0 && (n_tiles & 3) == 0 && wn->kv_len >= 4 * BN;
+      if (carry) {
+        const int64_t next_first = ((int64_t)wn->kv_start - w->kv_start) * ROWB;  // from this chunk's first tile
+        kpast_delta = vpast_delta = next_first - (int64_t)n_tiles * TILE;
+        past_stride = TILE;
       }
-    if (h == 0) {
-      const float lse = (l > 0.f) ? (ms[qb] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
-      a.lse_part[slot_rows + (int64_t)bh * a.S + row_g] = lse;
+    }
+    if (!carry) {
+      kpast_delta = vpast_delta = -(int64_t)TILE;
+      past_stride = 0;
+    }
+
+    if (!carried) {
+      if (it > 0) __syncthreads();  // every wave is done with the ring slots of the previous chunk
+      // the first tiles go out next to the Q loads: one memory latency for all of them
+      issue_k(0, kChecked);
+      if (n_tiles > 1) issue_k(1, kChecked);
+      if (n_tiles > 2) issue_k(2, kChecked);
+      issue_v(0, kChecked);
+      if (n_tiles > 1) issue_v(1, kChecked);
+      __builtin_amdgcn_s_waitcnt(0);  // retire the Q loads with a wait the compiler can see (and the tiles)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      qk(s_even, 0);
+    }
+    // (carried: K(0) was consumed by the last block of the previous chunk, which left the
+    // scores of tile 0 in s_even; K(1), K(2), V(0), V(1) are in flight)
+    {
+      float cand[QB];
+      mask_tile(s_even, 0, kUnchecked);
+      tile_maxes(s_even, cand);
+      set_reference(cand);
+    }
+
+    // Steady blocks come in groups of four (ring slots are compile-time constants).  A group
+    // starting at u computes the scores of tiles u+1 .. u+4 and loads up to tile u+6:
+    //   plain groups   while those four tiles need no mask; without any mask in the chunk the last
+    //                  group runs up to tile n_tiles-1 and its last block computes the scores of
+    //                  the tile after the last one (the next chunk's first, or nothing of use);
+    //   masked groups  (diagonal chunks) for the rest: every block masks its tile u+1;
+    //   a chunk with surplus keys in its last tile keeps clear of that tile (its loads need the
+    //   clamped form) and leaves the rest to the general blocks.
+    const bool ragged = kv_tail >= 0;
+    const int plain_end = ragged ? min(first_masked, kv_tail - 2) : (diag ? first_masked : n_tiles + 1);
+    const int masked_end = (diag && !ragged) ? n_tiles + 1 : 0;
+    int u = 0;
+    for (; u + 4 < plain_end; u += 4) {
+      block(C0{}, std::true_type{}, std::false_type{}, u);
+      block(C1{}, std::true_type{}, std::false_type{}, u + 1);
+      block(C2{}, std::true_type{}, std::false_type{}, u + 2);
+      block(C3{}, std::true_type{}, std::false_type{}, u + 3);
+    }
+    for (; u + 4 < masked_end; u += 4) {
+      block(C0{}, std::true_type{}, std::true_type{}, u);
+      block(C1{}, std::true_type{}, std::true_type{}, u + 1);
+      block(C2{}, std::true_type{}, std::true_type{}, u + 2);
+      block(C3{}, std::true_type{}, std::true_type{}, u + 3);
+    }
+    for (; u < n_tiles; ++u) {
+      if (u & 1) block(C1{}, std::false_type{}, std::false_type{}, u);
+      else block(C0{}, std::false_type{}, std::false_type{}, u);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next chunk's first tiles, or re-reads of the last tile
+    if (carry) {
+      __syncthreads();
+      synced = true;
+    }
+
+    emit_partial(w);
+    reset_state();
+    carried = carry;
+  }
+
+  // ---- fused merge: this workgroup's rows over the partials it has just written.  The same
+  // arithmetic, in the same order, as merge_row; only the loads are batched differently: a
+  // workgroup has just two waves per SIMD to hide their latency with, so all partial LSEs go
+  // through LDS in one sweep, and the partial O rows of two output rows and up to eight parts
+  // are in flight together.
+  if (a.fuse_merge) {
+    constexpr int TPR = D / 8;  // threads per row, 8 columns each
+    constexpr int ROWS = 256 / TPR;
+    constexpr int R = 2, G = 8;
+    static_assert(sizeof(smem) >= kMaxParts * BM * sizeof(float), "partial LSEs of a q tile fit the rings");
+    float* lse_s = (float*)smem;  // [n_items][BM]
+    const SegItem* its = a.items + seg.item_begin;
+    __syncthreads();  // the partial stores of all four waves have completed and are visible to them
+    for (int i = wave; i < n_items; i += 4) {
+      const int64_t prow = its[i].part_base + (int64_t)bh * its[i].part_bh_stride + qt * BM;
+#pragma unroll
+      for (int rr = lane; rr < BM; rr += 64)
+        lse_s[i * BM + rr] = (qt * BM + rr < q_len) ? a.lse_part[prow + rr] : -INFINITY;
+    }
+    __syncthreads();
+    const int c8 = tid % TPR;
+    const typename PartRow<HP>::ptr o_base = (typename PartRow<HP>::ptr)a.o_part + c8 * 8;
+#pragma unroll 1
+    for (int r0 = 0; r0 < BM; r0 += R * ROWS) {
+      int rl[R];
+      bool ok[R];
+      float mx[R], wsum[R], acc[R][8];
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        rl[j] = r0 + j * ROWS + tid / TPR;
+        ok[j] = qt * BM + rl[j] < q_len;
+        mx[j] = -INFINITY;
+        wsum[j] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
+      }
+      for (int i = 0; i < n_items; ++i)
+#pragma unroll
+        for (int j = 0; j < R; ++j) mx[j] = fmaxf(mx[j], lse_s[i * BM + rl[j]]);
+#pragma unroll 1
+      for (int i0 = 0; i0 < n_items; i0 += G) {
+        f32x4 x0[R][G], x1[R][G];
+#pragma unroll
+        for (int u = 0; u < G; ++u)
+          if (i0 + u < n_items) {
+            const int64_t prow = its[i0 + u].part_base + (int64_t)bh * its[i0 + u].part_bh_stride + qt * BM;
+#pragma unroll
+            for (int j = 0; j < R; ++j)
+              if (ok[j]) PartRow<HP>::ld(o_base + (prow + rl[j]) * D, x0[j][u], x1[j][u]);
+          }
+#pragma unroll
+        for (int u = 0; u < G; ++u)
+          if (i0 + u < n_items) {
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+              const float L = lse_s[(i0 + u) * BM + rl[j]];
+              if (!ok[j] || L == -INFINITY) continue;  // identity element: its O may hold anything
+              const float w = __expf(L - mx[j]);
+              wsum[j] += w;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                acc[j][e] = __builtin_fmaf(w, x0[j][u][e], acc[j][e]);
+                acc[j][4 + e] = __builtin_fmaf(w, x1[j][u][e], acc[j][4 + e]);
+              }
+            }
+          }
+      }
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        if (!ok[j]) continue;
+        if (mx[j] != -INFINITY) {
+          const float inv = 1.f / wsum[j];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[j][e] *= inv;
+        }
+        const int64_t out_row = (int64_t)bh * a.S + q_start + qt * BM + rl[j];
+        Store8<DT>::st((char*)a.out + (out_row * D + c8 * 8) * 2, acc[j]);
+        if (c8 == 0) a.lse[out_row] = (mx[j] == -INFINITY) ? -INFINITY : mx[j] + __logf(wsum[j]);
+      }
     }
   }
 }
 
 // ---- merge ------------------------------------------------------------------------
-template <int DT> struct Store8;
-template <> struct Store8<0> {
-  static __device__ __forceinline__ void st(void* p, const float* x) {
-    f16x8 v;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = (_Float16)x[e];
-    *(f16x8*)p = v;
-  }
-};
-template <> struct Store8<1> {
-  static __device__ __forceinline__ void st(void* p, const float* x) {
-    bf16x8 v;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = (__bf16)x[e];
-    *(bf16x8*)p = v;
-  }
-};
-
-// 8 consecutive columns of one partial row as floats
-template <bool HP> struct PartRow;
-template <> struct PartRow<false> {
-  using ptr = const float*;
-  static __device__ __forceinline__ void ld(ptr p, f32x4& x0, f32x4& x1) {
-    x0 = *(const f32x4*)p;
-    x1 = *(const f32x4*)(p + 4);
-  }
-};
-template <> struct PartRow<true> {
-  using ptr = const _Float16*;
-  static __device__ __forceinline__ void ld(ptr p, f32x4& x0, f32x4& x1) {
-    const f16x8 v = *(const f16x8*)p;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      x0[e] = (float)v[e];
-      x1[e] = (float)v[4 + e];
-    }
-  }
-};
-
 template <int DT, int D, bool HP>
 __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
   constexpr int TPR = D / 8;  // threads per row, 8 columns each
   constexpr int ROWS = 256 / TPR;
-  int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / TPR;
-  if (row >= a.rows) return;
-  row = (row / a.sel_len) * a.S + a.sel_start + row % a.sel_len;
-  const int c8 = threadIdx.x % TPR;
-  // active slots of these rows: the set bits of a.active, visited in ascending order
-  const float* lse_row = a.lse_parts + row;
-  const typename PartRow<HP>::ptr o_row = (typename PartRow<HP>::ptr)a.o_parts + row * D + c8 * 8;
-  const int64_t lse_stride = a.part_stride_rows, o_stride = a.part_stride_rows * D;
-
-  float mx = -INFINITY;
-  for (uint64_t rest = a.active; rest; rest &= rest - 1) mx = fmaxf(mx, lse_row[__builtin_ctzll(rest) * lse_stride]);
-  float acc[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-  float wsum = 0.f;
-  if (mx != -INFINITY) {
-    // four slots per iteration: all their loads are issued before the first is consumed
-    uint64_t rest = a.active;
-    while (__builtin_popcountll(rest) >= 4) {
-      float L[4];
-      f32x4 x0[4], x1[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int64_t s = __builtin_ctzll(rest);
-        rest &= rest - 1;
-        L[u] = lse_row[s * lse_stride];
-        PartRow<HP>::ld(o_row + s * o_stride, x0[u], x1[u]);
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const float w = __expf(L[u] - mx);
-        if (L[u] == -INFINITY) continue;  // identity element: its O may hold anything
-        wsum += w;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          acc[e] = __builtin_fmaf(w, x0[u][e], acc[e]);
-          acc[4 + e] = __builtin_fmaf(w, x1[u][e], acc[4 + e]);
-        }
-      }
-    }
-    for (; rest; rest &= rest - 1) {
-      const int64_t s = __builtin_ctzll(rest);
-      const float Ls = lse_row[s * lse_stride];
-      const float w = __expf(Ls - mx);
-      f32x4 x0, x1;
-      PartRow<HP>::ld(o_row + s * o_stride, x0, x1);
-      if (Ls == -INFINITY) continue;
-      wsum += w;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        acc[e] = __builtin_fmaf(w, x0[e], acc[e]);
-        acc[4 + e] = __builtin_fmaf(w, x1[e], acc[4 + e]);
-      }
-    }
-    const float inv = 1.f / wsum;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] *= inv;
-  }
-  Store8<DT>::st((char*)a.out + (row * D + c8 * 8) * 2, acc);
-  if (c8 == 0) a.lse[row] = (mx == -INFINITY) ? -INFINITY : mx + __logf(wsum);
+  const MergeRegion reg = a.regions ? a.regions[blockIdx.y] : a.single;
+  const int64_t idx = (int64_t)blockIdx.x * ROWS + threadIdx.x / TPR;  // over heads x reg.len
+  if (idx >= (int64_t)a.heads * reg.len) return;
+  const int64_t row = (idx / reg.len) * a.S + reg.start + idx % reg.len;
+  SlotParts parts{reg.active, row, a.part_stride_rows};
+  merge_row<DT, D, HP>(parts, a.o_parts, a.lse_parts, a.out, a.lse, row, threadIdx.x % TPR);
 }
 
-// ---- item table from kernel arguments ------------------------------------------------
-__global__ __launch_bounds__(64) void write_items_kernel(const ItemPack pack, int n, WorkItem* dst) {
+// ---- segment + item table from kernel arguments -------------------------------------
+__global__ __launch_bounds__(64) void write_table_kernel(const TablePack pack, int n, Segment* seg_dst, SegItem* item_dst) {
   const int i = threadIdx.x;
-  if (i < n) dst[i] = pack.items[i];
+  if (i < n) item_dst[i] = pack.items[i];
+  if (i == 0) *seg_dst = pack.seg;
 }
 
 // ---- host launchers -----------------------------------------------------------------
-hipError_t launch_block_step(const BlockStepArgs& a, int dtype, int dim, hipStream_t stream) {
-  if (a.n_items <= 0) return hipSuccess;
+hipError_t launch_block(const BlockArgs& a, int dtype, int dim, hipStream_t stream) {
+  if (a.n_segs <= 0) return hipSuccess;
   const int q_tiles = a.q_tiles_max;
-  const int64_t groups = (int64_t)(a.n_items | 1) * a.BH;  // odd item count, see the kernel
-  const int64_t blocks = ((groups + 7) / 8) * 8 * q_tiles;
+  const int64_t groups = (int64_t)a.n_segs * a.BH;
+  const int64_t blocks = (a.groups ? (int64_t)a.groups_per_xcd : (groups + 7) / 8) * 8 * q_tiles;
   if (q_tiles <= 0 || blocks > INT32_MAX) return hipErrorInvalidValue;
   const unsigned grid = (unsigned)blocks;
 #define RA_LAUNCH_BLOCK(DT_, D_)                                                            \
@@ -641,17 +845,18 @@ hipError_t launch_block_step(const BlockStepArgs& a, int dtype, int dim, hipStre
   return hipGetLastError();
 }
 
-hipError_t launch_write_items(const ItemPack& pack, int n, WorkItem* dst, hipStream_t stream) {
-  if (n <= 0) return hipSuccess;
-  if (n > kMaxParts) return hipErrorInvalidValue;
-  write_items_kernel<<<1, 64, 0, stream>>>(pack, n, dst);
+hipError_t launch_write_table(const TablePack& pack, int n, Segment* seg_dst, SegItem* item_dst, hipStream_t stream) {
+  if (n <= 0 || n > kMaxParts) return hipErrorInvalidValue;
+  write_table_kernel<<<1, 64, 0, stream>>>(pack, n, seg_dst, item_dst);
   return hipGetLastError();
 }
 
 hipError_t launch_merge(const MergeArgs& a, int dtype, int dim, hipStream_t stream) {
-  if (a.rows <= 0) return hipSuccess;
+  if (a.n_regions <= 0 || a.max_len <= 0 || a.heads <= 0) return hipSuccess;
   const int rows_per_block = 256 / (dim / 8);
-  const unsigned grid = (unsigned)((a.rows + rows_per_block - 1) / rows_per_block);
+  const int64_t cols = ((int64_t)a.heads * a.max_len + rows_per_block - 1) / rows_per_block;
+  if (cols > INT32_MAX || a.n_regions > 65535) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)cols, (unsigned)a.n_regions);
 #define RA_LAUNCH_MERGE(DT_, D_)                                                 \
   do {                                                                        \
     if (a.half_partials) merge_kernel<DT_, D_, true><<<grid, 256, 0, stream>>>(a);  \

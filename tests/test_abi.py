@@ -81,6 +81,26 @@ def test_parameter_validation(ralib):
     assert wb(None) == 0
 
 
+def test_workspace_counts_only_visible_steps(ralib):
+    # one partial row per query row and VISIBLE ring step: causal ranks hold r + 1 steps, not npes
+    wb = ralib.ringattn_workspace_bytes
+    row = (128 + 1) * 4
+    dense = wb(ctypes.byref(params(npes=8, seqlen=(4096,) * 8, dim=128, heads=32, causal=0)))
+    causal = wb(ctypes.byref(params(npes=8, seqlen=(4096,) * 8, dim=128, heads=32, causal=1)))
+    assert dense == 8 * 32 * 32768 * row
+    assert causal == 36 * 32 * 4096 * row and causal * 64 == dense * 36       # 36 of the 64 (rank, step) pairs
+    # zigzag: the low half of rank r sees r + 1 steps, the high half all 8: (36 + 64) / 2 of 64 chunk-steps
+    zig = wb(ctypes.byref(params(npes=8, seqlen=(4096,) * 8, dim=128, heads=32, causal=1, layout=1)))
+    assert zig == (36 + 64) * 32 * 2048 * row
+    # fp16 partials (flag 4): 2 dim + 4 bytes per partial row
+    half = wb(ctypes.byref(params(npes=8, seqlen=(4096,) * 8, dim=128, heads=32, causal=1, flags=4)))
+    assert half == 36 * 32 * 4096 * (2 * 128 + 4)
+    # ragged, unequal ranks
+    lens = (100, 333, 1, 77)
+    ragged = wb(ctypes.byref(params(npes=4, seqlen=lens, dim=64, causal=1)))
+    assert ragged == sum((r + 1) * n for r, n in enumerate(lens)) * (64 + 1) * 4
+
+
 def test_plan_lifetime_with_caller_workspace(ralib):
     # a caller-provided workspace needs no HIP call, so the plan life cycle runs on a CPU host
     p = params()
