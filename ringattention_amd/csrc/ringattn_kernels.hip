@@ -222,6 +222,175 @@ static __device__ __forceinline__ void merge_row(Parts parts, const void* o_part
   if (c8 == 0) lse[out_row] = (mx == -INFINITY) ? -INFINITY : mx + __logf(wsum);
 }
 
+// workgroup -> job (segment, head, q tile); false for the holes of the grid.  blockIdx mod 8 is
+// the XCD: the q tiles of a (segment, head) group are consecutive workgroups of one XCD and share
+// its K and V in that L2.  With a group table the host has dealt the heads to the XCDs and
+// listed, per XCD, the segments of one head after the other (busiest first): ranks of a head
+// follow each other through the same K and V, which then stay in that XCD's L2 / the
+// memory-side cache.  Without one, groups are dealt to the XCDs in segment-major order.
+static __device__ __forceinline__ bool decode_job(const BlockArgs& a, Segment& seg, int& bh, int& qt) {
+  const int q_tiles = a.q_tiles_max;
+  const int xcd = blockIdx.x & 7, wslot = blockIdx.x >> 3;
+  int sg;
+  if (a.groups) {
+    const int2 g = a.groups[xcd * a.groups_per_xcd + wslot / q_tiles];
+    sg = g.x;
+    bh = g.y;
+    if (sg < 0) return false;
+  } else {
+    const int group = (wslot / q_tiles) * 8 + xcd;
+    if (group >= a.n_segs * a.BH) return false;
+    sg = group / a.BH;
+    bh = group % a.BH;
+  }
+  seg = a.segs[sg];
+  qt = wslot % q_tiles;
+  if (qt * kBlockM >= seg.q_len) return false;  // segments shorter than the longest one
+  if (seg.reverse_tiles) qt = (seg.q_len + kBlockM - 1) / kBlockM - 1 - qt;  // most keys first
+  return true;
+}
+
+// ---- merge of one job's rows (128 rows of a segment, one head) over the partials of the
+// segment's items.  The same arithmetic, in the same order, as merge_row; only the loads are
+// arranged differently: the block kernel, which runs this at the end of a workgroup, has just two
+// waves per SIMD to hide memory latency with, and every round trip it waits for is time its
+// compute unit runs half empty.  So all partial LSEs are fetched in one sweep and parked in LDS
+// (lse_s: [items][128] floats), and the partial O rows move in batches of 256 bytes per thread
+// (two output rows x four or eight parts), three batches in flight at any time.
+typedef __attribute__((address_space(3))) float lds_float;
+template <int DT, int D, bool HP>
+static __device__ __forceinline__ void merge_job_rows(const void* o_part, const float* lse_part, void* out, float* lse,
+                                                      const SegItem* items, const Segment& seg, int bh, int qt, int S,
+                                                      lds_float* lse_s) {
+  constexpr int BM = kBlockM;
+  constexpr int TPR = D / 8;  // threads per row, 8 columns each
+  constexpr int ROWS = 256 / TPR;
+  constexpr int R = 2, G = HP ? 8 : 4;  // rows per thread and parts per batch: 64 registers a batch
+  constexpr int RSTEP = R * ROWS;
+  constexpr int KMAX = kMaxParts / 4;  // parts per wave in the LSE sweep
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n_parts = seg.item_count;
+  const SegItem* its = items + seg.item_begin;
+  const int row0 = qt * BM;  // first row of the job within the segment
+  __syncthreads();  // the partial stores of all four waves have completed and are visible to them; the LDS is idle
+  {
+    float v[KMAX][2];
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      const int i = wave + 4 * k;
+      if (i < n_parts) {
+        const int64_t prow = its[i].part_base + (int64_t)bh * its[i].part_bh_stride + row0;
+        v[k][0] = (row0 + lane < seg.q_len) ? lse_part[prow + lane] : -INFINITY;
+        v[k][1] = (row0 + lane + 64 < seg.q_len) ? lse_part[prow + lane + 64] : -INFINITY;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      const int i = wave + 4 * k;
+      if (i < n_parts) {
+        lse_s[i * BM + lane] = v[k][0];
+        lse_s[i * BM + lane + 64] = v[k][1];
+      }
+    }
+  }
+  __syncthreads();
+  const int c8 = tid % TPR, rsub = tid / TPR;
+  // this thread's 8 columns of a partial row: 16 bytes as fp16, 32 as fp32
+  constexpr int PB = HP ? 16 : 32;
+  constexpr int NV = PB / 16;
+  const char* o_base = (const char*)o_part + c8 * PB;
+  const int n_groups = (n_parts + G - 1) / G;
+  const int n_batches = (BM / RSTEP) * n_groups;  // batch b: rows of b / n_groups, parts of b % n_groups
+  struct Batch {
+    f32x4 raw[R][G][NV];  // as loaded; fp16 partials are widened when they are used
+  };
+  auto row_of = [&](int b, int j) { return (b / n_groups) * RSTEP + j * ROWS + rsub; };  // within the job
+  auto fetch = [&](int b, Batch& t) {
+    const int i0 = (b % n_groups) * G;
+#pragma unroll
+    for (int u = 0; u < G; ++u)
+      if (i0 + u < n_parts) {
+        const int64_t prow = its[i0 + u].part_base + (int64_t)bh * its[i0 + u].part_bh_stride + row0;
+#pragma unroll
+        for (int j = 0; j < R; ++j)
+          if (row0 + row_of(b, j) < seg.q_len) {
+            const char* src = o_base + (prow + row_of(b, j)) * (D * (PB / 8));
+#pragma unroll
+            for (int v = 0; v < NV; ++v) t.raw[j][u][v] = *(const f32x4*)(src + 16 * v);
+          }
+      }
+  };
+  float mx[R], wsum[R], acc[R][8];
+  auto accumulate = [&](int b, const Batch& t) {
+    const int g = b % n_groups, i0 = g * G;
+    if (g == 0) {  // new rows: L = max over the parts first
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        mx[j] = -INFINITY;
+        wsum[j] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
+      }
+      for (int i = 0; i < n_parts; ++i)
+#pragma unroll
+        for (int j = 0; j < R; ++j) mx[j] = fmaxf(mx[j], lse_s[i * BM + row_of(b, j)]);
+    }
+#pragma unroll
+    for (int u = 0; u < G; ++u)
+      if (i0 + u < n_parts) {
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          const float L = lse_s[(i0 + u) * BM + row_of(b, j)];
+          if (row0 + row_of(b, j) >= seg.q_len || L == -INFINITY) continue;  // identity element: its O may hold anything
+          const float w = __expf(L - mx[j]);
+          wsum[j] += w;
+          float x[8];
+          if (HP) {
+            const f16x8 hv = __builtin_bit_cast(f16x8, t.raw[j][u][0]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = (float)hv[e];
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              x[e] = t.raw[j][u][0][e];
+              x[4 + e] = t.raw[j][u][NV - 1][e];
+            }
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[j][e] = __builtin_fmaf(w, x[e], acc[j][e]);
+        }
+      }
+    if (g == n_groups - 1) {  // all parts in: normalise and store
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        if (row0 + row_of(b, j) >= seg.q_len) continue;
+        if (mx[j] != -INFINITY) {
+          const float inv = 1.f / wsum[j];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[j][e] *= inv;
+        }
+        const int64_t out_row = (int64_t)bh * S + seg.q_start + row0 + row_of(b, j);
+        Store8<DT>::st((char*)out + (out_row * D + c8 * 8) * 2, acc[j]);
+        if (c8 == 0) lse[out_row] = (mx[j] == -INFINITY) ? -INFINITY : mx[j] + __logf(wsum[j]);
+      }
+    }
+  };
+  // three batches in flight
+  Batch t0, t1, t2;
+  fetch(0, t0);
+  if (1 < n_batches) fetch(1, t1);
+#pragma unroll 1
+  for (int b = 0; b < n_batches; b += 3) {
+    if (b + 2 < n_batches) fetch(b + 2, t2);
+    accumulate(b, t0);
+    if (b + 3 < n_batches) fetch(b + 3, t0);
+    if (b + 1 < n_batches) accumulate(b + 1, t1);
+    if (b + 4 < n_batches) fetch(b + 4, t1);
+    if (b + 2 < n_batches) accumulate(b + 2, t2);
+  }
+}
+
 // ---- block attention: the ring steps of 128 query rows ----------------------------------
 // A KV chunk is consumed in 32-key tiles held in two 4-deep LDS rings (K and V), filled by
 // direct-to-LDS loads that run two blocks ahead.  Block u of the loop runs, in ONE
@@ -259,32 +428,10 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockArgs
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 31, h = lane >> 5;
 
-  // workgroup -> (segment, head, q tile).  blockIdx mod 8 is the XCD: the q tiles of a
-  // (segment, head) group stay on one XCD and share its K and V in that L2.  Groups are
-  // segment-major and the host lists the segments by decreasing work, so the workgroups that
-  // are dispatched last are the short ones.
-  // With a group table the host has dealt the heads to the XCDs and listed, per XCD, the
-  // segments of one head after the other: ranks of a head follow each other through the same
-  // K and V, which then stay in that XCD's L2 / the memory-side cache.
-  const int q_tiles = a.q_tiles_max;
-  const int xcd = blockIdx.x & 7, wslot = blockIdx.x >> 3;
-  int sg, bh;
-  if (a.groups) {
-    const int2 g = a.groups[xcd * a.groups_per_xcd + wslot / q_tiles];
-    sg = g.x;
-    bh = g.y;
-    if (sg < 0) return;
-  } else {
-    const int group = (wslot / q_tiles) * 8 + xcd;
-    if (group >= a.n_segs * a.BH) return;
-    sg = group / a.BH;
-    bh = group % a.BH;
-  }
-  const Segment seg = a.segs[sg];
+  Segment seg;
+  int bh, qt;
+  if (!decode_job(a, seg, bh, qt)) return;
   const int q_start = seg.q_start, q_len = seg.q_len;
-  int qt = wslot % q_tiles;
-  if (qt * BM >= q_len) return;  // segments shorter than the longest one
-  if (seg.reverse_tiles) qt = (q_len + BM - 1) / BM - 1 - qt;  // most keys first
   const int n_items = seg.item_count;
   // items in run order: table order, except that item `last_item` is moved to the end
   auto item_at = [&](int i) -> const SegItem* {
@@ -720,86 +867,11 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockArgs
     carried = carry;
   }
 
-  // ---- fused merge: this workgroup's rows over the partials it has just written.  The same
-  // arithmetic, in the same order, as merge_row; only the loads are batched differently: a
-  // workgroup has just two waves per SIMD to hide their latency with, so all partial LSEs go
-  // through LDS in one sweep, and the partial O rows of two output rows and up to eight parts
-  // are in flight together.
+  // ---- fused merge: this workgroup's rows over the partials it has just written
   if (a.fuse_merge) {
-    constexpr int TPR = D / 8;  // threads per row, 8 columns each
-    constexpr int ROWS = 256 / TPR;
-    constexpr int R = 2, G = 8;
     static_assert(sizeof(smem) >= kMaxParts * BM * sizeof(float), "partial LSEs of a q tile fit the rings");
-    float* lse_s = (float*)smem;  // [n_items][BM]
-    const SegItem* its = a.items + seg.item_begin;
-    __syncthreads();  // the partial stores of all four waves have completed and are visible to them
-    for (int i = wave; i < n_items; i += 4) {
-      const int64_t prow = its[i].part_base + (int64_t)bh * its[i].part_bh_stride + qt * BM;
-#pragma unroll
-      for (int rr = lane; rr < BM; rr += 64)
-        lse_s[i * BM + rr] = (qt * BM + rr < q_len) ? a.lse_part[prow + rr] : -INFINITY;
-    }
-    __syncthreads();
-    const int c8 = tid % TPR;
-    const typename PartRow<HP>::ptr o_base = (typename PartRow<HP>::ptr)a.o_part + c8 * 8;
-#pragma unroll 1
-    for (int r0 = 0; r0 < BM; r0 += R * ROWS) {
-      int rl[R];
-      bool ok[R];
-      float mx[R], wsum[R], acc[R][8];
-#pragma unroll
-      for (int j = 0; j < R; ++j) {
-        rl[j] = r0 + j * ROWS + tid / TPR;
-        ok[j] = qt * BM + rl[j] < q_len;
-        mx[j] = -INFINITY;
-        wsum[j] = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
-      }
-      for (int i = 0; i < n_items; ++i)
-#pragma unroll
-        for (int j = 0; j < R; ++j) mx[j] = fmaxf(mx[j], lse_s[i * BM + rl[j]]);
-#pragma unroll 1
-      for (int i0 = 0; i0 < n_items; i0 += G) {
-        f32x4 x0[R][G], x1[R][G];
-#pragma unroll
-        for (int u = 0; u < G; ++u)
-          if (i0 + u < n_items) {
-            const int64_t prow = its[i0 + u].part_base + (int64_t)bh * its[i0 + u].part_bh_stride + qt * BM;
-#pragma unroll
-            for (int j = 0; j < R; ++j)
-              if (ok[j]) PartRow<HP>::ld(o_base + (prow + rl[j]) * D, x0[j][u], x1[j][u]);
-          }
-#pragma unroll
-        for (int u = 0; u < G; ++u)
-          if (i0 + u < n_items) {
-#pragma unroll
-            for (int j = 0; j < R; ++j) {
-              const float L = lse_s[(i0 + u) * BM + rl[j]];
-              if (!ok[j] || L == -INFINITY) continue;  // identity element: its O may hold anything
-              const float w = __expf(L - mx[j]);
-              wsum[j] += w;
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                acc[j][e] = __builtin_fmaf(w, x0[j][u][e], acc[j][e]);
-                acc[j][4 + e] = __builtin_fmaf(w, x1[j][u][e], acc[j][4 + e]);
-              }
-            }
-          }
-      }
-#pragma unroll
-      for (int j = 0; j < R; ++j) {
-        if (!ok[j]) continue;
-        if (mx[j] != -INFINITY) {
-          const float inv = 1.f / wsum[j];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) acc[j][e] *= inv;
-        }
-        const int64_t out_row = (int64_t)bh * a.S + q_start + qt * BM + rl[j];
-        Store8<DT>::st((char*)a.out + (out_row * D + c8 * 8) * 2, acc[j]);
-        if (c8 == 0) a.lse[out_row] = (mx[j] == -INFINITY) ? -INFINITY : mx[j] + __logf(wsum[j]);
-      }
-    }
+    merge_job_rows<DT, D, HP>(a.o_part, a.lse_part, a.out, a.lse, a.items, seg, bh, qt, a.S,
+                              (lds_float*)(__attribute__((address_space(3))) void*)smem);
   }
 }
 
