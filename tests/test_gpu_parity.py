@@ -4,9 +4,12 @@ inputs.  Tolerances are the ones the engine is specified with:
     O   : max-abs error <= 1e-2 against the float64 oracle (O is stored in fp16 / bf16)
     LSE : relative error <= 1e-3 (fp32)
 
-Large workloads are compared on a seeded sample of rows (the first rows of the sequence,
-where causal rows see few keys and |O| is largest, are always included) and through
-size-independent properties on the full output."""
+Large workloads are compared on whole heads (cfg2 in full; one or two complete heads of cfg3 and
+cfg4; complete q tiles at chunk starts, middles and ends of cfg5) plus a seeded sample of rows
+(the first rows of the sequence, where causal rows see few keys and |O| is largest, are always
+included), and through size-independent properties on the full output.  Where the storage type's
+own half unit in the last place exceeds 1e-2 (bf16 values of magnitude 4 and more), that half
+unit is the bound: see check_rows."""
 import math
 import os
 
@@ -48,22 +51,74 @@ def sample_rows(w, n, seed=0):
     return np.unique(np.concatenate([rng.integers(0, w.rows, n), first, last_head, chunk_edges]))
 
 
-def check_rows(oracle, w, q, k, v, out, lse, rows, scale=None):
+def storage_ulp(x, dtype):
+    """Spacing of the storage type at |x| (numpy array, float64)."""
+    mant, emin = (10, -14) if dtype == "fp16" else (7, -126)
+    e = np.floor(np.log2(np.maximum(np.abs(x), 2.0 ** emin)))
+    return 2.0 ** (e - mant)
+
+
+def check_rows(oracle, w, q, k, v, out, lse, rows, scale=None, half_partials=None):
+    """O against the float64 oracle: max-abs error <= 1e-2 -- or half a unit in the last place of the
+    storage type where that is more (a bf16 value in [4, 8) is a multiple of 2^-5, so even the correctly
+    rounded result can be 1.56e-2 off; only the first rows of a causal sequence, which average very few
+    V rows, get that large) -- and within ONE unit in the last place (of the row's largest element) of the
+    oracle rounded to the storage type (two with fp16 per-step partials).  LSE: relative error <= 1e-3."""
     o_ref, l_ref = oracle.attention_rows(q, k, v, w.dtype, causal=w.causal, rows=rows, scale=scale)
     idx = torch.from_numpy(rows).cuda()
     o_gpu = out.reshape(-1, w.dim)[idx].double().cpu().numpy()
     l_gpu = lse.reshape(-1)[idx].double().cpu().numpy()
     assert np.isfinite(o_gpu).all() and np.isfinite(l_gpu).all()
-    err_o = np.abs(o_gpu - o_ref).max()
+    ulp = storage_ulp(o_ref, w.dtype)
+    tol = np.maximum(O_TOL, 0.5 * ulp)
+    err = np.abs(o_gpu - o_ref)
+    err_o = err.max()
     err_l = (np.abs(l_gpu - l_ref) / np.maximum(np.abs(l_ref), 1e-3)).max()
     # also against the oracle rounded to the storage type (what a perfect kernel would store)
     o_rounded = bits_to_float64(float32_to_bits(o_ref.astype(np.float32), w.dtype), w.dtype)
-    err_r = np.abs(o_gpu - o_rounded).max()
-    print(f"parity {w.name}: {len(rows)} rows, max|dO| = {err_o:.3e} vs fp64, {err_r:.3e} vs rounded fp64, "
-          f"max rel dLSE = {err_l:.3e}, max|O| = {np.abs(o_ref).max():.2f}")
-    assert err_o <= O_TOL, f"{w.name}: max|dO| = {err_o:.3e}"
+    err_r = np.abs(o_gpu - o_rounded)
+    # ... measured in units in the last place of the ROW's largest element: the kernel rounds the
+    # probabilities to the storage type before the PV product (as the reference does,
+    # csrc/ring_attention.cu:604), which moves every element of a row by about that much however
+    # small the element itself is
+    ulp_r = storage_ulp(np.maximum(np.abs(o_gpu), np.abs(o_rounded)).max(axis=1, keepdims=True), w.dtype)
+    print(f"parity {w.name}: {len(rows)} rows, max|dO| = {err_o:.3e} vs fp64, {err_r.max():.3e} vs rounded fp64 "
+          f"({(err_r / ulp_r).max():.2f} ulp), max rel dLSE = {err_l:.3e}, max|O| = {np.abs(o_ref).max():.2f}, "
+          f"{int((tol > O_TOL).sum())} elements where half an ulp exceeds 1e-2")
+    assert (err <= tol).all(), f"{w.name}: max|dO| = {err_o:.3e}, worst excess {(err - tol).max():.3e}"
+    # fp16 per-step partials (RINGATTN_FLAG_HALF_PARTIALS) round once more on the way: two units then
+    ulps = 2 if (w.half_partials if half_partials is None else half_partials) else 1
+    assert (err_r <= ulps * ulp_r).all(), f"{w.name}: {(err_r / ulp_r).max():.2f} ulp from the rounded oracle"
     assert err_l <= LSE_RTOL, f"{w.name}: max rel dLSE = {err_l:.3e}"
     return err_o, err_l
+
+
+def whole_head_rows(w, heads):
+    """All rows of the given flat head indices (b * H + h)."""
+    return np.concatenate([np.arange(h * w.seq, (h + 1) * w.seq) for h in heads])
+
+
+def workload_rows(w):
+    """Rows compared for each of the five workloads: whole heads where the oracle gets through them
+    in seconds, complete 128-row q tiles at the start, middle and end of chunks for the longest one,
+    plus the seeded sample (first rows of the sequence, last head, chunk edges)."""
+    bh = w.batch * w.heads
+    if w.name == "cfg2":
+        rows = np.arange(w.rows)                                        # everything
+    elif w.name == "cfg3":
+        rows = np.concatenate([whole_head_rows(w, [bh - 1]), sample_rows(w, 512)])
+    elif w.name == "cfg4":
+        rows = np.concatenate([whole_head_rows(w, [0, bh - 1]), sample_rows(w, 384)])
+    elif w.name == "cfg5":
+        tiles = []
+        for head, chunk, where in ((0, 0, 0), (0, 3, w.chunk // 2), (5, 7, w.chunk - 128), (bh - 1, w.npes - 1, w.chunk - 128),
+                                   (bh - 1, 8, 0), (9, 15, 4096 + 128)):
+            first = head * w.seq + chunk * w.chunk + where
+            tiles.append(np.arange(first, first + 128))
+        rows = np.concatenate(tiles + [sample_rows(w, 1400)])
+    else:
+        rows = sample_rows(w, 256)
+    return np.unique(rows)
 
 
 def test_cfg1_full_against_oracle_and_golden(oracle):
@@ -85,12 +140,12 @@ def test_causal_small_golden(oracle):
     assert np.abs(out.float().cpu().numpy() - g["o_f32"]).max() <= O_TOL
 
 
-@pytest.mark.parametrize("name,nrows", [("cfg2", 2048), ("cfg3", 512), ("cfg4", 384), ("cfg5", 96)])
-def test_workload_sampled_rows(oracle, name, nrows):
+@pytest.mark.parametrize("name", ["cfg2", "cfg3", "cfg4", "cfg5"])
+def test_workload_whole_heads(oracle, name):
     w = WORKLOADS[name]
     q, k, v = api.make_qkv_bits(w)
     out, lse = forward(w, q, k, v)
-    check_rows(oracle, w, q, k, v, out, lse, sample_rows(w, nrows))
+    check_rows(oracle, w, q, k, v, out, lse, workload_rows(w))
     # full-size properties: finite everywhere, convexity |O| <= max|V| (O is an average of V rows)
     assert torch.isfinite(out).all() and torch.isfinite(lse).all()
     vmax = np.abs(bits_to_float64(v, w.dtype)).max()
@@ -289,13 +344,18 @@ def test_zigzag_cfg4_sampled_rows(oracle):
     torch.cuda.synchronize()
     plan.close()
     assert torch.isfinite(out).all() and torch.isfinite(lse).all()
-    rows_seq = sample_rows(w, 384)                                  # (head, sequence position) pairs
+    # (head, sequence position) pairs: the whole of head 17 and the seeded sample
+    rows_seq = np.unique(np.concatenate([whole_head_rows(w, [17]), sample_rows(w, 384)]))
     head, posn = rows_seq // w.seq, rows_seq % w.seq
     rows_mem = torch.from_numpy(head * w.seq + inv[posn]).cuda()
     o_ref, l_ref = oracle.attention_rows(q, k, v, w.dtype, causal=True, rows=rows_seq)
     o_gpu = out.reshape(-1, w.dim)[rows_mem].double().cpu().numpy()
     l_gpu = lse.reshape(-1)[rows_mem].double().cpu().numpy()
-    assert np.abs(o_gpu - o_ref).max() <= O_TOL
+    ulp = storage_ulp(o_ref, w.dtype)
+    assert (np.abs(o_gpu - o_ref) <= np.maximum(O_TOL, 0.5 * ulp)).all()      # the rule of check_rows
+    o_rounded = bits_to_float64(float32_to_bits(o_ref.astype(np.float32), w.dtype), w.dtype)
+    assert (np.abs(o_gpu - o_rounded) <= storage_ulp(np.maximum(np.abs(o_gpu), np.abs(o_rounded)).max(axis=1, keepdims=True),
+                                                      w.dtype)).all()
     assert (np.abs(l_gpu - l_ref) / np.maximum(np.abs(l_ref), 1e-3)).max() <= LSE_RTOL
 
 
@@ -555,7 +615,8 @@ def test_half_precision_partials(oracle, w, layout):
     torch.cuda.synchronize()
     # same parity bar against the oracle, and close to the fp32-partial result: each merged part
     # carries at most half an fp16 ulp of max |V|, plus one ulp of the output type
-    check_rows(oracle, w, q, k, v, o16[:, :, inv].contiguous(), l16[:, :, inv].contiguous(), np.arange(w.rows))
+    check_rows(oracle, w, q, k, v, o16[:, :, inv].contiguous(), l16[:, :, inv].contiguous(), np.arange(w.rows),
+               half_partials=True)
     vmax = np.abs(bits_to_float64(v, w.dtype)).max()
     ulp_out = 2.0**-10 if w.dtype == "fp16" else 2.0**-7
     assert (o16.float() - o32.float()).abs().max().item() <= vmax * 2.0**-11 + ulp_out * vmax

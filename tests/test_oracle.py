@@ -143,6 +143,75 @@ def test_ring_partials_follow_the_ring_schedule(oracle):
             assert np.abs(po[x, s] - scipy.special.softmax(logits) @ vf[sl]).max() < 1e-14
 
 
+def test_causal_ring_partials_against_scipy(oracle):
+    # causal ring, unequal chunks: rank r at step s meets chunk j = (r + s) mod P; j > r gives no
+    # partial (LSE -inf), j == r the keys up to the row's own position, j < r the whole chunk
+    rng = np.random.default_rng(14)
+    seqlen, d = [12, 20, 8, 16], 8
+    P, S = len(seqlen), sum(seqlen)
+    start = np.concatenate([[0], np.cumsum(seqlen)])
+    q, k, v = (rand_bits(rng, (1, 2, S, d), "bf16") for _ in range(3))
+    rows = np.arange(2 * S)
+    o, lse, po, pl = oracle.ring_rows(q, k, v, "bf16", seqlen, rows, causal=True, tile=5, want_parts=True)
+    qf, kf, vf = (bits_to_float64(x, "bf16") for x in (q, k, v))
+    for x in rows:
+        h, pos = divmod(int(x), S)
+        r = int(np.searchsorted(start, pos, side="right") - 1)
+        seen = 0
+        for s in range(P):
+            j = (r + s) % P
+            if j > r:
+                assert pl[x, s] == -np.inf
+                continue
+            hi = pos + 1 if j == r else start[j + 1]
+            sl = slice(start[j], hi)
+            seen += hi - start[j]
+            logits = (kf[0, h, sl] @ qf[0, h, pos]) / math.sqrt(d)
+            assert abs(pl[x, s] - scipy.special.logsumexp(logits)) < 1e-13
+            assert np.abs(po[x, s] - scipy.special.softmax(logits) @ vf[0, h, sl]).max() < 1e-14
+        assert seen == pos + 1                    # the visible steps cover keys 0..pos exactly once
+    # and the merged rows equal plain causal attention
+    o_ref, lse_ref = torch_attention(q, k, v, "bf16", causal=True)
+    assert np.abs(o - o_ref.reshape(-1, d)).max() < 1e-13 and np.abs(lse - lse_ref.reshape(-1)).max() < 1e-12
+
+
+def test_block_partial_with_a_shifted_diagonal_against_scipy(oracle):
+    # mask_mode 1 with diag_offset: key t visible to row i iff t <= i + diag_offset
+    rng = np.random.default_rng(15)
+    cq, ck, d, off = 10, 24, 16, 7
+    q = rand_bits(rng, (cq, d), "fp16")
+    k, v = (rand_bits(rng, (ck, d), "fp16") for _ in range(2))
+    o, lse = oracle.block_partial(q, k, v, "fp16", mask_mode=1, diag_offset=off, tile=6)
+    qf, kf, vf = (bits_to_float64(x, "fp16") for x in (q, k, v))
+    for i in range(cq):
+        logits = (kf[:i + off + 1] @ qf[i]) / math.sqrt(d)
+        assert abs(lse[i] - scipy.special.logsumexp(logits)) < 1e-13
+        assert np.abs(o[i] - scipy.special.softmax(logits) @ vf[:i + off + 1]).max() < 1e-14
+
+
+def test_ring_rows_with_rounded_probabilities(oracle):
+    # round_p: the PV product uses p rounded to the storage type, the row sum the unrounded p.
+    # Rebuilt here with numpy on ONE tile per chunk (then the max is the chunk max and p = softmax numerators).
+    rng = np.random.default_rng(16)
+    P, c, d = 3, 16, 8
+    q, k, v = (rand_bits(rng, (1, 1, P * c, d), "bf16") for _ in range(3))
+    rows = np.array([0, 7, c + 2, 2 * c + 15])
+    o, lse, po, pl = oracle.ring_rows(q, k, v, "bf16", [c] * P, rows, tile=c, round_p=True, want_parts=True)
+    o_exact, lse_exact = oracle.ring_rows(q, k, v, "bf16", [c] * P, rows, tile=c)
+    assert np.array_equal(lse, lse_exact)                     # sums come from the unrounded p
+    qf, kf, vf = (bits_to_float64(x, "bf16")[0, 0] for x in (q, k, v))
+    for x, row in enumerate(rows):
+        r = row // c
+        for s in range(P):
+            j = (r + s) % P
+            logits = (kf[j * c:(j + 1) * c] @ qf[row]) / math.sqrt(d)
+            p = np.exp(logits - logits.max())
+            p_rounded = bits_to_float64(float32_to_bits(p.astype(np.float32), "bf16"), "bf16")
+            want = p_rounded @ vf[j * c:(j + 1) * c] / p.sum()
+            assert np.abs(po[x, s] - want).max() < 1e-6       # p passes through float32 on its way to bf16 here
+    assert 0 < np.abs(o - o_exact).max() < 2e-2
+
+
 def test_block_partial_matches_library_and_rounding_of_p_is_small(oracle):
     rng = np.random.default_rng(6)
     c, d = 48, 32
