@@ -11,7 +11,8 @@ import shutil
 import subprocess
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "liboracle.so")
+# ORACLE_LIB: load another build instead (the sanitized one of tests/test_sanitizers.py)
+LIB_PATH = os.environ.get("ORACLE_LIB") or os.path.join(HERE, "liboracle.so")
 
 
 def build_oracle():
@@ -26,6 +27,19 @@ def build_oracle():
         raise RuntimeError("gcc failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
     os.replace(tmp, LIB_PATH)
     return LIB_PATH
+
+
+def build_oracle_sanitized(clang, out_dir):
+    """The oracle with AddressSanitizer + UndefinedBehaviorSanitizer, built with the clang whose
+    sanitizer runtime the sanitized library uses as well (one runtime per process); no OpenMP."""
+    out = os.path.join(out_dir, "liboracle_san.so")
+    cmd = [clang, "-O1", "-g", "-fPIC", "-shared", "-std=c11", "-fsanitize=address,undefined",
+           "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer", "-shared-libsan",
+           os.path.join(HERE, "attention_oracle.c"), "-o", out, "-lm"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("clang failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
+    return out
 
 
 if __name__ == "__main__":

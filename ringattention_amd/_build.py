@@ -7,7 +7,8 @@ import subprocess
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_DIR = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
-LIB_PATH = os.path.join(PKG_DIR, "libringattn.so")
+# RINGATTN_LIB: load another build of the library instead (the sanitized host build of the CPU tests)
+LIB_PATH = os.environ.get("RINGATTN_LIB") or os.path.join(PKG_DIR, "libringattn.so")
 
 TORCH_LIB_PATH = os.path.join(PKG_DIR, "libringattn_torch.so")
 
@@ -64,18 +65,35 @@ def build_torch_shim(verbose=False):
     return TORCH_LIB_PATH
 
 
-PROBE_PATH = os.path.join(PKG_DIR, "issue_rate_probe")
+def sanitizer_runtime():
+    """Path of the AddressSanitizer runtime of hipcc's clang (to be preloaded into a python that
+    loads a sanitized library)."""
+    clang = os.path.join(os.path.dirname(os.path.realpath(shutil.which("hipcc") or "/opt/rocm/bin/hipcc")), "..",
+                         "lib", "llvm", "bin", "clang")
+    if not os.path.exists(clang):
+        clang = "/opt/rocm/lib/llvm/bin/clang"
+    res = subprocess.run([clang, "--print-file-name=libclang_rt.asan-x86_64.so"], capture_output=True, text=True)
+    path = res.stdout.strip()
+    if res.returncode != 0 or not os.path.isabs(path) or not os.path.exists(path):
+        raise RuntimeError("AddressSanitizer runtime of hipcc's clang not found")
+    return clang, path
 
 
-def build_probe():
-    """Compile csrc/issue_rate_probe.hip, the stand-alone instruction-mix micro-benchmark."""
+def build_sanitized_library(out_dir):
+    """The library with its HOST code (validation, schedule, plan lifetime, data generator, launch
+    stubs) under AddressSanitizer and UndefinedBehaviorSanitizer, for the CPU tests.  The sanitizer
+    flags are given to the host compilation only (-Xarch_host); the device code is the usual one."""
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    cmd = [hipcc, "--offload-arch=gfx950", "-O2", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           os.path.join(CSRC, "issue_rate_probe.hip"), "-o", PROBE_PATH]
+    out = os.path.join(out_dir, "libringattn_san.so")
+    cmd = [hipcc] + [f for f in HIPCC_FLAGS if f != "-O3"] + [
+        "-O1", "-g", "-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+        "-Xarch_host", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer", "-shared-libsan",
+        "-I", os.path.join(REPO_DIR, "include"), "-I", CSRC]
+    cmd += [os.path.join(CSRC, s) for s in SOURCES] + ["-o", out]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
-    return PROBE_PATH
+    return out
 
 
 HARNESS_PATH = os.path.join(PKG_DIR, "reference_harness")
@@ -94,6 +112,5 @@ def build_harness():
 
 if __name__ == "__main__":
     print(build_library(verbose=True))
-    print(build_probe())
     print(build_harness())
     print(build_torch_shim(verbose=True))
