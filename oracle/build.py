@@ -26,7 +26,23 @@ def build_oracle():
     if res.returncode != 0:
         raise RuntimeError("gcc failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
     os.replace(tmp, LIB_PATH)
+    with open(LIB_PATH + ".stamp", "w") as f:
+        f.write(source_id() + "\n")
     return LIB_PATH
+
+
+def source_id():
+    import hashlib
+    with open(os.path.join(HERE, "attention_oracle.c"), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()
+
+
+def is_current():
+    stamp = LIB_PATH + ".stamp"
+    if not (os.path.exists(LIB_PATH) and os.path.exists(stamp)):
+        return False
+    with open(stamp) as f:
+        return f.read().strip() == source_id()
 
 
 def build_oracle_sanitized(clang, out_dir):

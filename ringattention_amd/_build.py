@@ -21,6 +21,35 @@ HIPCC_FLAGS = [
 ]
 
 
+def source_id(paths):
+    """sha256 over the given files: what a build product was made from."""
+    import hashlib
+    h = hashlib.sha256()
+    for path in sorted(paths):
+        with open(path, "rb") as f:
+            h.update(os.path.basename(path).encode() + b"\0" + f.read())
+    return h.hexdigest()
+
+
+def library_sources():
+    return [os.path.join(CSRC, s) for s in SOURCES] + [os.path.join(CSRC, "ringattn_kernels.h"),
+                                                       os.path.join(REPO_DIR, "include", "ringattn.h")]
+
+
+def is_current(product, sources):
+    """True if `product` exists and its stamp file names exactly these sources' contents."""
+    stamp = product + ".stamp"
+    if not (os.path.exists(product) and os.path.exists(stamp)):
+        return False
+    with open(stamp) as f:
+        return f.read().strip() == source_id(sources)
+
+
+def write_stamp(product, sources):
+    with open(product + ".stamp", "w") as f:
+        f.write(source_id(sources) + "\n")
+
+
 def build_library(verbose=False):
     """Compile every HIP source of the package into libringattn.so.  Always recompiles."""
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
@@ -35,7 +64,16 @@ def build_library(verbose=False):
     if verbose:
         print(res.stderr)
     os.replace(tmp, LIB_PATH)
+    write_stamp(LIB_PATH, library_sources())
     return LIB_PATH
+
+
+def torch_shim_sources():
+    return [os.path.join(CSRC, "ringattn_torch.cpp"), os.path.join(REPO_DIR, "include", "ringattn.h")]
+
+
+def harness_sources():
+    return [os.path.join(CSRC, "reference_harness.cpp"), os.path.join(REPO_DIR, "include", "ringattn.h")]
 
 
 def build_torch_shim(verbose=False):
@@ -62,6 +100,7 @@ def build_torch_shim(verbose=False):
     if verbose:
         print(res.stderr)
     os.replace(tmp, TORCH_LIB_PATH)
+    write_stamp(TORCH_LIB_PATH, torch_shim_sources())
     return TORCH_LIB_PATH
 
 
@@ -107,6 +146,7 @@ def build_harness():
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
+    write_stamp(HARNESS_PATH, harness_sources())
     return HARNESS_PATH
 
 

@@ -32,14 +32,33 @@ def _ptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
-def _check_tensor(t, name, dtype=None):
-    # conventions of include/attention_api.cuh:12-18: device-resident and contiguous
+def _check_meta(t, name, dtype=None, shape=None):
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} must have shape {tuple(shape)}, not {tuple(t.shape)}")
+    if dtype is not None and t.dtype != dtype:
+        raise ValueError(f"{name} must have dtype {dtype}")
+
+
+def _check_place(t, name):
     if not t.is_cuda:
         raise ValueError(f"{name} must be a device tensor")
     if not t.is_contiguous():
         raise ValueError(f"{name} must be contiguous")
-    if dtype is not None and t.dtype != dtype:
-        raise ValueError(f"{name} must have dtype {dtype}")
+
+
+def _check_tensors(*specs):
+    """specs: (tensor, name, dtype or None, shape or None).  Shapes and dtypes of ALL tensors against
+    what the plan expects first (the C ABI sees raw pointers only: a wrongly sized buffer would become
+    an out-of-bounds access on the device), then the conventions of include/attention_api.cuh:12-18:
+    device-resident and contiguous."""
+    for t, name, dtype, shape in specs:
+        _check_meta(t, name, dtype, shape)
+    for t, name, _, _ in specs:
+        _check_place(t, name)
+
+
+def _check_tensor(t, name, dtype=None, shape=None):
+    _check_tensors((t, name, dtype, shape))
 
 
 def make_params(npes, seqlen, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, flags=0,
@@ -55,13 +74,14 @@ class RingAttention:
     """A forward plan for P virtual ring ranks on one GPU."""
 
     def __init__(self, npes, chunk, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, graph=False,
-                 kv_heads=0, layout="contiguous", timing=False, half_partials=False):
+                 kv_heads=0, layout="contiguous", timing=False, half_partials=False, workspace=None):
         """`chunk`: tokens per rank -- one int for equal chunks or a list of npes lengths
         (the per-PE seqlen[] of csrc/ring_attention.cu:753).  `kv_heads`: heads of K and V for
         grouped-query attention (0 = same as `heads`).  `layout`: "contiguous" (rank r holds
         the tokens after those of rank r-1) or "zigzag" (rank r holds a low and a high
         half-chunk; see zigzag_order).  `half_partials`: keep the per-step partial O in fp16
-        (half the workspace and merge traffic; needs |V| < 65504)."""
+        (half the workspace and merge traffic; needs |V| < 65504).  `workspace`: a (device address,
+        bytes) pair the caller owns and keeps alive, instead of an allocation by the plan."""
         self.lib = _lib.load()
         self.seqlen = [int(chunk)] * npes if isinstance(chunk, int) else [int(x) for x in chunk]
         if len(self.seqlen) != npes:
@@ -78,7 +98,8 @@ class RingAttention:
                                   | (FLAG_HALF_PARTIALS if half_partials else 0), kv_heads,
                                   LAYOUT_CODE[layout])
         self.handle = ctypes.c_void_p()
-        check(self.lib.ringattn_plan_create(ctypes.byref(self.params), None, 0, ctypes.byref(self.handle)),
+        ws_ptr, ws_bytes = (None, 0) if workspace is None else (ctypes.c_void_p(int(workspace[0])), int(workspace[1]))
+        check(self.lib.ringattn_plan_create(ctypes.byref(self.params), ws_ptr, ws_bytes, ctypes.byref(self.handle)),
               "ringattn_plan_create")
 
     def close(self):
@@ -95,30 +116,33 @@ class RingAttention:
     def _shape(self):
         return (self.batch, self.heads, self.seq, self.dim)
 
-    def forward(self, q, k, v, out=None, lse=None, stream=None):
+    def _qkv_specs(self, q, k, v):
         kv_shape = (self.batch, self.kv_heads, self.seq, self.dim)
-        for t, nm, shp in ((q, "q", self._shape()), (k, "k", kv_shape), (v, "v", kv_shape)):
-            _check_tensor(t, nm, self.torch_dtype)
-            if tuple(t.shape) != shp:
-                raise ValueError(f"{nm} must have shape {shp}")
+        return [(q, "q", self.torch_dtype, self._shape()), (k, "k", self.torch_dtype, kv_shape),
+                (v, "v", self.torch_dtype, kv_shape)]
+
+    def forward(self, q, k, v, out=None, lse=None, stream=None):
+        _check_tensors(*self._qkv_specs(q, k, v))
         if out is None:
             out = torch.empty_like(q)
         if lse is None:
-            lse = torch.empty((self.batch, self.heads, self.seq), dtype=torch.float32, device=q.device)
-        _check_tensor(out, "out", self.torch_dtype)
-        _check_tensor(lse, "lse", torch.float32)
+            lse = torch.empty(self._shape()[:3], dtype=torch.float32, device=q.device)
+        _check_tensors((out, "out", self.torch_dtype, self._shape()), (lse, "lse", torch.float32, self._shape()[:3]))
         check(self.lib.ringattn_fwd(self.handle, _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _stream_ptr(stream)),
               "ringattn_fwd")
         return out, lse
 
     def block_forward(self, step, q, k, v, o_part=None, lse_part=None, stream=None):
-        for t, nm in ((q, "q"), (k, "k"), (v, "v")):
-            _check_tensor(t, nm, self.torch_dtype)
+        specs = self._qkv_specs(q, k, v)
+        if o_part is not None:
+            specs.append((o_part, "o_part", self.part_dtype, self._shape()))
+        if lse_part is not None:
+            specs.append((lse_part, "lse_part", torch.float32, self._shape()[:3]))
+        _check_tensors(*specs)
         if o_part is None:
             o_part = torch.zeros(self._shape(), dtype=self.part_dtype, device=q.device)
-        _check_tensor(o_part, "o_part", self.part_dtype)
         if lse_part is None:
-            lse_part = torch.full((self.batch, self.heads, self.seq), float("-inf"), dtype=torch.float32, device=q.device)
+            lse_part = torch.full(self._shape()[:3], float("-inf"), dtype=torch.float32, device=q.device)
         check(self.lib.ringattn_block_fwd(self.handle, int(step), _ptr(q), _ptr(k), _ptr(v), _ptr(o_part),
                                           _ptr(lse_part), _stream_ptr(stream)), "ringattn_block_fwd")
         return o_part, lse_part
@@ -126,9 +150,17 @@ class RingAttention:
     def rank_step_forward(self, rank, step, q, k_chunk, v_chunk, o_part=None, lse_part=None, stream=None):
         """One ring step of one rank on rank-local tensors (q: the rank's rows; k_chunk, v_chunk: the
         chunk of rank (rank + step) % npes).  Returns the rank-local partial (O, LSE)."""
-        rows = self.seqlen[rank]
-        for t, nm in ((q, "q"), (k_chunk, "k_chunk"), (v_chunk, "v_chunk")):
-            _check_tensor(t, nm, self.torch_dtype)
+        if not (0 <= rank < self.npes and 0 <= step < self.npes):
+            raise ValueError("rank and step must be in [0, npes)")
+        rows, kv_rows = self.seqlen[rank], self.seqlen[(rank + step) % self.npes]
+        specs = [(q, "q", self.torch_dtype, (self.batch, self.heads, rows, self.dim)),
+                 (k_chunk, "k_chunk", self.torch_dtype, (self.batch, self.kv_heads, kv_rows, self.dim)),
+                 (v_chunk, "v_chunk", self.torch_dtype, (self.batch, self.kv_heads, kv_rows, self.dim))]
+        if o_part is not None:
+            specs.append((o_part, "o_part", self.part_dtype, (self.batch, self.heads, rows, self.dim)))
+        if lse_part is not None:
+            specs.append((lse_part, "lse_part", torch.float32, (self.batch, self.heads, rows)))
+        _check_tensors(*specs)
         if o_part is None:
             o_part = torch.zeros((self.batch, self.heads, rows, self.dim), dtype=self.part_dtype, device=q.device)
         if lse_part is None:
@@ -139,13 +171,17 @@ class RingAttention:
 
     def rank_merge(self, rank, o_parts, lse_parts, out=None, lse=None, stream=None):
         """Merge of one rank's per-step partials [npes, B, H, rows, d] / [npes, B, H, rows]."""
+        if not 0 <= rank < self.npes:
+            raise ValueError("rank must be in [0, npes)")
         rows = self.seqlen[rank]
-        _check_tensor(o_parts, "o_parts", self.part_dtype)
-        _check_tensor(lse_parts, "lse_parts", torch.float32)
+        _check_tensors((o_parts, "o_parts", self.part_dtype, (self.npes, self.batch, self.heads, rows, self.dim)),
+                       (lse_parts, "lse_parts", torch.float32, (self.npes, self.batch, self.heads, rows)))
         if out is None:
             out = torch.empty((self.batch, self.heads, rows, self.dim), dtype=self.torch_dtype, device=o_parts.device)
         if lse is None:
             lse = torch.empty((self.batch, self.heads, rows), dtype=torch.float32, device=o_parts.device)
+        _check_tensor(out, "out", self.torch_dtype, (self.batch, self.heads, rows, self.dim))
+        _check_tensor(lse, "lse", torch.float32, (self.batch, self.heads, rows))
         check(self.lib.ringattn_rank_merge(self.handle, int(rank), _ptr(o_parts), _ptr(lse_parts), _ptr(out), _ptr(lse),
                                            _stream_ptr(stream)), "ringattn_rank_merge")
         return out, lse
@@ -178,12 +214,14 @@ class RingAttention:
 
     def merge_ring(self, o_parts, lse_parts, out=None, lse=None, stream=None):
         """Ring-aware merge of caller-held per-step partials [npes, B, H, S, d] / [npes, B, H, S]."""
-        _check_tensor(o_parts, "o_parts", self.part_dtype)
-        _check_tensor(lse_parts, "lse_parts", torch.float32)
+        _check_tensors((o_parts, "o_parts", self.part_dtype, (self.npes,) + self._shape()),
+                       (lse_parts, "lse_parts", torch.float32, (self.npes,) + self._shape()[:3]))
         if out is None:
             out = torch.empty(self._shape(), dtype=self.torch_dtype, device=o_parts.device)
         if lse is None:
-            lse = torch.empty((self.batch, self.heads, self.seq), dtype=torch.float32, device=o_parts.device)
+            lse = torch.empty(self._shape()[:3], dtype=torch.float32, device=o_parts.device)
+        _check_tensor(out, "out", self.torch_dtype, self._shape())
+        _check_tensor(lse, "lse", torch.float32, self._shape()[:3])
         check(self.lib.ringattn_merge_ring(self.handle, _ptr(o_parts), _ptr(lse_parts), _ptr(out), _ptr(lse),
                                            _stream_ptr(stream)), "ringattn_merge_ring")
         return out, lse
@@ -210,15 +248,27 @@ def zigzag_order(seqlen):
 def merge(o_parts, lse_parts, dtype, stream=None):
     """n-way (O, LSE) merge.  o_parts [n, rows, d] fp32, lse_parts [n, rows] fp32."""
     lib = _lib.load()
-    _check_tensor(o_parts, "o_parts", torch.float32)
-    _check_tensor(lse_parts, "lse_parts", torch.float32)
+    if o_parts.dim() != 3:
+        raise ValueError("o_parts must be [n_parts, rows, dim]")
     n, rows, d = o_parts.shape
+    _check_tensors((o_parts, "o_parts", torch.float32, None), (lse_parts, "lse_parts", torch.float32, (n, rows)))
     code = DTYPE_CODE[dtype]
     out = torch.empty((rows, d), dtype=TORCH_DTYPE[code], device=o_parts.device)
     lse = torch.empty((rows,), dtype=torch.float32, device=o_parts.device)
     check(lib.ringattn_merge(_ptr(o_parts), _ptr(lse_parts), n, rows, d, code, _ptr(out), _ptr(lse), _stream_ptr(stream)),
           "ringattn_merge")
     return out, lse
+
+
+def _check_rank_call(q, k, v, out, lse, npes, mype, seqlen, dim):
+    if len(seqlen) != npes or not 0 <= mype < npes:
+        raise ValueError("seqlen must hold npes lengths and mype must be in [0, npes)")
+    rows, total = int(seqlen[mype]), int(sum(seqlen))
+    specs = [(q, "q", None, (rows, dim)), (k, "k", q.dtype, (total, dim)), (v, "v", q.dtype, (total, dim)),
+             (out, "out", q.dtype, (rows, dim))]
+    if lse is not None:
+        specs.append((lse, "lse", torch.float32, (rows,)))
+    _check_tensors(*specs)
 
 
 def ring_attention(q, k, v, out, npes, mype, seqlen, dim, max_seq, lse=None, causal=False, softmax_scale=0.0):
@@ -228,8 +278,7 @@ def ring_attention(q, k, v, out, npes, mype, seqlen, dim, max_seq, lse=None, cau
     chunks, out [seqlen[mype], dim].  Blocks until done, like the reference (:721).
     """
     lib = _lib.load()
-    for t, nm in ((q, "q"), (k, "k"), (v, "v"), (out, "out")):
-        _check_tensor(t, nm, q.dtype)
+    _check_rank_call(q, k, v, out, lse, npes, mype, seqlen, dim)
     arr = (ctypes.c_int * len(seqlen))(*[int(x) for x in seqlen])
     check(lib.ringattn_ring_attention(_ptr(q), _ptr(k), _ptr(v), _ptr(out),
                                       _ptr(lse) if lse is not None else None, int(npes), int(mype), arr, int(dim),
@@ -243,8 +292,7 @@ def ring_attention_noalloc(q, k, v, out, npes, mype, seqlen, dim, max_seq, lse=N
     """ring_attention() through the entry point that allocates nothing (static device scratch);
     asynchronous on `stream`.  Raises RingattnError (workspace) if the rank's partials do not fit."""
     lib = _lib.load()
-    for t, nm in ((q, "q"), (k, "k"), (v, "v"), (out, "out")):
-        _check_tensor(t, nm, q.dtype)
+    _check_rank_call(q, k, v, out, lse, npes, mype, seqlen, dim)
     arr = (ctypes.c_int * len(seqlen))(*[int(x) for x in seqlen])
     check(lib.ringattn_ring_attention_noalloc(_ptr(q), _ptr(k), _ptr(v), _ptr(out),
                                               _ptr(lse) if lse is not None else None, int(npes), int(mype), arr,

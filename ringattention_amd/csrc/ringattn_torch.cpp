@@ -3,13 +3,15 @@
 // CHECK_CUDA / CHECK_CONTIGUOUS / CHECK_INPUT, :8-18, but the reference never builds one).
 // Registers   ringattn::fwd(q, k, v, seqlen, causal, softmax_scale, zigzag) -> (out, lse)
 // with the dispatcher.  Only plumbing lives here: tensor checks, output allocation, the
-// current stream, a cache of plans; all computation is ringattn_fwd of libringattn.so.
+// current stream, a bounded cache of plans (one per parameter set and stream); all computation is
+// ringattn_fwd of libringattn.so.
 #include <ATen/ATen.h>
 #include <c10/hip/HIPGuard.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/library.h>
 
 #include <map>
+#include <memory>
 #include <mutex>
 #include <tuple>
 #include <vector>
@@ -25,21 +27,49 @@ namespace {
   RA_CHECK_DEVICE(x);     \
   RA_CHECK_CONTIGUOUS(x)
 
-// Plans are created once per distinct parameter set and device and kept until the process
-// ends (the workspace of a plan is what makes a forward allocation-free).
-using PlanKey = std::tuple<int, std::vector<int>, int, int, int, int, int, int, int, float, int>;
-std::mutex g_mu;
-std::map<PlanKey, ringattn_plan*> g_plans;
-
-ringattn_plan* plan_for(const PlanKey& key, const ringattn_params& p) {
-  std::lock_guard<std::mutex> lk(g_mu);
-  auto it = g_plans.find(key);
-  if (it != g_plans.end()) return it->second;
+// A plan owns ONE workspace and is meant for one forward at a time, so the cache holds a plan
+// per (parameter set, device, STREAM): forwards on different streams never share partials, and
+// forwards on one stream are ordered by the stream.  A per-plan mutex keeps two host threads
+// from enqueueing on the same plan at once.  The cache is bounded: beyond kMaxPlans the least
+// recently used plan that nobody is enqueueing on is destroyed (its workspace goes back to the
+// device); hipFree inside ringattn_plan_destroy waits for the work that still uses it.
+using PlanKey = std::tuple<int, void*, std::vector<int>, int, int, int, int, int, int, int, float>;
+struct Entry {
   ringattn_plan* plan = nullptr;
-  const int rc = ringattn_plan_create(&p, nullptr, 0, &plan);
-  TORCH_CHECK(rc == RINGATTN_OK, "ringattn_plan_create: ", ringattn_strerror(rc));
-  g_plans.emplace(key, plan);
-  return plan;
+  std::mutex mu;  // held while a forward is being enqueued on the plan
+  uint64_t last_use = 0;
+};
+constexpr size_t kMaxPlans = 16;
+std::mutex g_mu;
+std::map<PlanKey, std::shared_ptr<Entry>> g_plans;
+uint64_t g_clock = 0;
+
+std::shared_ptr<Entry> plan_for(const PlanKey& key, const ringattn_params& p) {
+  std::vector<std::shared_ptr<Entry>> evicted;
+  std::shared_ptr<Entry> e;
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_plans.find(key);
+    if (it != g_plans.end()) {
+      it->second->last_use = ++g_clock;
+      return it->second;
+    }
+    while (g_plans.size() >= kMaxPlans) {
+      auto victim = g_plans.end();
+      for (auto j = g_plans.begin(); j != g_plans.end(); ++j)
+        if (j->second.use_count() == 1 && (victim == g_plans.end() || j->second->last_use < victim->second->last_use)) victim = j;
+      if (victim == g_plans.end()) break;  // every plan is in use right now: grow
+      evicted.push_back(victim->second);
+      g_plans.erase(victim);
+    }
+    e = std::make_shared<Entry>();
+    const int rc = ringattn_plan_create(&p, nullptr, 0, &e->plan);
+    TORCH_CHECK(rc == RINGATTN_OK, "ringattn_plan_create: ", ringattn_strerror(rc));
+    e->last_use = ++g_clock;
+    g_plans.emplace(key, e);
+  }
+  for (auto& v : evicted) (void)ringattn_plan_destroy(v->plan);
+  return e;
 }
 
 std::tuple<at::Tensor, at::Tensor> fwd(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
@@ -77,14 +107,18 @@ std::tuple<at::Tensor, at::Tensor> fwd(const at::Tensor& q, const at::Tensor& k,
   p.kv_heads = (int)k.size(1) == p.heads ? 0 : (int)k.size(1);
   p.layout = zigzag ? RINGATTN_LAYOUT_ZIGZAG : RINGATTN_LAYOUT_CONTIGUOUS;
   const int device = q.device().index();
-  const PlanKey key{device, lens, p.dim, p.batch, p.heads, p.dtype, p.causal, p.kv_heads, p.layout, p.softmax_scale, 0};
-
   c10::hip::HIPGuard guard(device);  // plan creation allocates on the current device
-  ringattn_plan* plan = plan_for(key, p);
+  hipStream_t stream = c10::hip::getCurrentHIPStream(device).stream();
+  const PlanKey key{device, (void*)stream, lens, p.dim, p.batch, p.heads, p.dtype, p.causal, p.kv_heads, p.layout,
+                    p.softmax_scale};
+  std::shared_ptr<Entry> entry = plan_for(key, p);
   at::Tensor out = at::empty_like(q);
   at::Tensor lse = at::empty({q.size(0), q.size(1), q.size(2)}, q.options().dtype(at::kFloat));
-  const int rc = ringattn_fwd(plan, q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr<float>(),
-                              c10::hip::getCurrentHIPStream(device).stream());
+  int rc;
+  {
+    std::lock_guard<std::mutex> lk(entry->mu);
+    rc = ringattn_fwd(entry->plan, q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr<float>(), stream);
+  }
   TORCH_CHECK(rc == RINGATTN_OK, "ringattn_fwd: ", ringattn_strerror(rc));
   return {out, lse};
 }

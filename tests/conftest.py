@@ -33,17 +33,18 @@ def pytest_collection_modifyitems(config, items):
 
 @pytest.fixture(scope="session", autouse=True)
 def built_artifacts():
-    """The tests load what is built; only where a build product is missing altogether (a fresh
-    checkout) is it compiled here, once per session."""
+    """The tests load what is built.  A build product is compiled here, once per session, only where it
+    is missing or was made from other sources than the ones in the tree (every build leaves a stamp
+    with the hash of its sources): tests never run against a stale binary."""
     from ringattention_amd import _build
-    if not os.path.exists(_build.LIB_PATH):
+    if "RINGATTN_LIB" not in os.environ and not _build.is_current(_build.LIB_PATH, _build.library_sources()):
         _build.build_library()
-    if not os.path.exists(_build.TORCH_LIB_PATH):
+    if not _build.is_current(_build.TORCH_LIB_PATH, _build.torch_shim_sources()):
         _build.build_torch_shim()
-    if not os.path.exists(_build.HARNESS_PATH):
+    if not _build.is_current(_build.HARNESS_PATH, _build.harness_sources()):
         _build.build_harness()
     from oracle import build as oracle_build
-    if not os.path.exists(oracle_build.LIB_PATH):
+    if "ORACLE_LIB" not in os.environ and not oracle_build.is_current():
         oracle_build.build_oracle()
 
 

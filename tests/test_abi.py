@@ -289,3 +289,43 @@ def test_plans_from_many_threads(ralib):
     for t in threads:
         t.join()
     assert not errors, errors
+
+
+def test_python_front_end_refuses_wrongly_shaped_tensors(ralib):
+    # The C ABI takes raw pointers: every tensor is checked against the plan's geometry before the
+    # call, so a mis-sized buffer is a ValueError and never an out-of-bounds access on the device.
+    import torch
+    from ringattention_amd import api
+    P, c, d, B, H = 4, 128, 64, 2, 3
+    need = ralib.ringattn_workspace_bytes(ctypes.byref(params(npes=P, seqlen=(c,) * P, dim=d, batch=B, heads=H)))
+    plan = api.RingAttention(P, c, d, B, H, "fp16", False, workspace=(1 << 20, need))   # host only: never launched
+    S = P * c
+    good = torch.zeros(B, H, S, d, dtype=torch.float16)
+    with pytest.raises(ValueError, match="k must have shape"):
+        plan.forward(good, good[:, :, :-1], good)
+    with pytest.raises(ValueError, match="q must have dtype"):
+        plan.forward(good.float(), good, good)
+    with pytest.raises(ValueError, match="q must be a device tensor"):          # right shape, wrong place
+        plan.forward(good, good, good)
+    with pytest.raises(ValueError, match="o_part must have shape"):
+        plan.block_forward(0, good, good, good, o_part=torch.zeros(B, H, S - 1, d), lse_part=torch.zeros(B, H, S))
+    with pytest.raises(ValueError, match="k_chunk must have shape"):
+        plan.rank_step_forward(1, 2, good[:, :, :c], good[:, :, :c + 1], good[:, :, :c])
+    with pytest.raises(ValueError, match="rank and step"):
+        plan.rank_step_forward(P, 0, good[:, :, :c], good[:, :, :c], good[:, :, :c])
+    with pytest.raises(ValueError, match="lse_parts must have shape"):
+        plan.rank_merge(0, torch.zeros(P, B, H, c, d), torch.zeros(P, B, H, c + 1))
+    with pytest.raises(ValueError, match="o_parts must have shape"):
+        plan.merge_ring(torch.zeros(P - 1, B, H, S, d), torch.zeros(P, B, H, S))
+    with pytest.raises(ValueError, match="lse_parts must have shape"):
+        api.merge(torch.zeros(3, 64, d), torch.zeros(3, 65), "fp16")
+    q1 = torch.zeros(c, d, dtype=torch.float16)
+    kv = torch.zeros(S, d, dtype=torch.float16)
+    for entry in (api.ring_attention, api.ring_attention_noalloc):
+        with pytest.raises(ValueError, match="k must have shape"):
+            entry(q1, kv[:-1], kv, torch.zeros_like(q1), P, 0, [c] * P, d, c)
+        with pytest.raises(ValueError, match="out must have shape"):
+            entry(q1, kv, kv, torch.zeros(c + 1, d, dtype=torch.float16), P, 0, [c] * P, d, c)
+        with pytest.raises(ValueError, match="mype"):
+            entry(q1, kv, kv, torch.zeros_like(q1), P, P, [c] * P, d, c)
+    plan.close()
