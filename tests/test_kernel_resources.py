@@ -1,0 +1,88 @@
+"""What the compiler made of the block kernel: the d = 128 instantiations must keep two waves
+per SIMD (256 registers) and their steady key loops -- the loops that hold 64 MFMAs, four
+32-key blocks -- must not touch scratch memory.  (The kernel as a whole does spill a few values
+around the chunk prologue and the general, non-unrolled blocks; those run once per chunk.)
+Compiles the kernels to assembly for gfx950; needs hipcc but no GPU."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def loops_of(asm):
+    """(label, instructions) of every innermost loop of a function body: from the block the
+    compiler marks as the loop header to the last branch back to it (or to the block of wait
+    and barrier it sometimes places right in front of the header)."""
+    lines = asm.split("\n")
+    where = {}
+    for i, line in enumerate(lines):
+        m = re.match(r"^(\.LBB\d+_\d+):", line)
+        if m:
+            where[m.group(1)] = i
+    out = []
+    for i, line in enumerate(lines):
+        if "Inner Loop Header" not in line:
+            continue
+        head = max((k for k in where.values() if k <= i), default=None)
+        if head is None:
+            continue
+        targets = {lab for lab, k in where.items() if head - 12 <= k <= head}
+        last = None
+        for j in range(i + 1, len(lines)):
+            m = re.match(r"^\s*s_(?:cbranch_\w+|branch)\s+(\.LBB\d+_\d+)\s*$", lines[j])
+            if m and m.group(1) in targets:
+                last = j
+        if last is not None:
+            body = [l.strip() for l in lines[i + 1:last + 1]]
+            out.append((lines[head].split(":")[0], [l for l in body if l and not l.startswith((";", "."))]))
+    return out
+
+
+def test_steady_key_loops_are_spill_free_at_two_waves_per_simd(tmp_path):
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc")
+    from ringattention_amd import _build
+    src = os.path.join(_build.CSRC, "ringattn_kernels.hip")
+    out = tmp_path / "kernels.s"
+    flags = [f for f in _build.HIPCC_FLAGS if f not in ("-shared", "-fPIC", "-pthread")]
+    res = subprocess.run([hipcc] + flags + ["-S", "--cuda-device-only", "-Rpass-analysis=kernel-resource-usage",
+                                            "-I", os.path.join(ROOT, "include"), "-I", _build.CSRC, src, "-o", str(out)],
+                         capture_output=True, text=True, timeout=900)
+    assert res.returncode == 0, res.stderr[-2000:]
+    # occupancy and register count from the compiler's remarks
+    usage = {}
+    name = None
+    for line in res.stderr.split("\n"):
+        m = re.search(r"Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+            usage[name] = {}
+        for key in ("VGPRs", "ScratchSize [bytes/lane]", "Occupancy [waves/SIMD]", "LDS Size [bytes/block]"):
+            m = re.search(re.escape(key) + r": (\d+)", line)
+            if m and name:
+                usage[name][key] = int(m.group(1))
+    blocks = {n: u for n, u in usage.items() if "block_attention_kernel" in n}
+    assert len(blocks) == 8                                    # {fp16, bf16} x {64, 128} x {fp32, fp16 partials}
+    for n, u in blocks.items():
+        assert u["Occupancy [waves/SIMD]"] == 2, (n, u)
+        assert u["VGPRs"] <= 256, (n, u)
+        if "Li128E" in n:
+            assert u["LDS Size [bytes/block]"] == 65536, (n, u)   # two workgroups per compute unit
+    asm = out.read_text()
+    checked = 0
+    for n in blocks:
+        if "Li128E" not in n:
+            continue
+        start = asm.index("\n" + n + ":")
+        end = asm.index(".amdhsa_kernel " + n, start)
+        steady = [(lab, ins) for lab, ins in loops_of(asm[start:end]) if sum(i.startswith("v_mfma") for i in ins) == 64]
+        assert len(steady) == 2, (n, len(steady))              # the plain and the masked groups of four blocks
+        for lab, ins in steady:
+            assert not any(i.startswith("scratch_") for i in ins), (n, lab)
+            checked += 1
+    assert checked == 8
