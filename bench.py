@@ -2,14 +2,17 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4]
 
-A step is one full forward of the workload: every ring step of every virtual rank and the merge
-of the per-step partials (one block-attention launch, the merge fused at the end of each
-workgroup), with Q/K/V already resident in HBM.  Prints one JSON line.  `value` is algorithmic TFLOP/s (4*B*H*d*visible
-(q,k) pairs per forward) over the wall time of K steps; `roofline` prices the
-block-attention launch of the same forward against the dense MFMA peak, timed by an
-event pair on the launch stream (a second pass of K forwards on a plan with the timing
-flag); `merge` times the merge kernel alone against HBM bandwidth; `cpu_baseline` is the
-CPU oracle timed on this host on a bounded sample of the same workload's rows.
+A step is one full forward of the workload: every ring step of every virtual rank, with Q/K/V
+already resident in HBM -- one block-attention launch in which a workgroup walks all ring steps
+of its 128 query rows with the softmax state in registers and writes O and LSE at the end.
+Prints one JSON line.  `value` is algorithmic TFLOP/s (4*B*H*d*visible (q,k) pairs per forward)
+over the wall time of K steps; `roofline` prices the block-attention launch of the same forward
+against the dense MFMA peak, timed by an event pair on the launch stream (a second pass of K
+forwards on a plan with the timing flag); `forward_with_step_partials` is the same forward on a
+plan that keeps the ring steps apart (a partial (O, LSE) per step, merged at the end of each
+workgroup; --step-partials makes that one the headline); `merge` times the merge kernel alone, on
+caller-held per-step partials, against HBM bandwidth; `cpu_baseline` is the CPU oracle timed on
+this host on a bounded sample of the same workload's rows.
 """
 import argparse
 import json
@@ -64,6 +67,9 @@ def main():
     ap.add_argument("--rank-local", action="store_true",
                     help="also time the ring rank by rank on rank-local buffers (one launch per rank and step)")
     ap.add_argument("--per-step", action="store_true", help="also time one block-attention launch per ring step")
+    ap.add_argument("--step-partials", action="store_true",
+                    help="time the forward that keeps the ring steps apart (per-step partials in a workspace, merged at "
+                         "the end) instead of the one that carries the softmax state through the steps")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the cpu_baseline sample (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -81,7 +87,7 @@ def main():
     q, k, v = api.make_qkv_bits(w)
     qd, kd, vd = (api.bits_to_tensor(x, w.dtype) for x in (q, k, v))
     plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=w.graph, layout=args.layout,
-                             half_partials=w.half_partials)
+                             half_partials=w.half_partials, step_partials=args.step_partials)
     out = torch.empty_like(qd)
     lse = torch.empty((w.batch, w.heads, w.seq), dtype=torch.float32, device="cuda")
     stream = torch.cuda.current_stream()
@@ -106,9 +112,9 @@ def main():
     peak = PEAK_TFLOPS[w.dtype]
     # ---- block kernel: the same forward on a plan that records an event pair around its
     # block-attention launch, on the stream it is launched on.  The launch is the whole ring (every
-    # step of every rank, the merge of a workgroup's rows fused at its end).
+    # step of every rank).
     timed = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=False,
-                              layout=args.layout, timing=True, half_partials=w.half_partials)
+                              layout=args.layout, timing=True, half_partials=w.half_partials, step_partials=args.step_partials)
     timed.forward(qd, kd, vd, out, lse, stream)
     launch_ms = []
     for _ in range(args.steps):
@@ -119,7 +125,7 @@ def main():
     avg_launch_ms = float(launch_ms.mean())
     block_tflops = w.flops / n_launch / (avg_launch_ms * 1e-3) / 1e12
     traffic, traffic_source = None, "not measured for this workload / layout"
-    if args.layout == "contiguous" and w.name in MEASURED_TRAFFIC:
+    if args.layout == "contiguous" and not args.step_partials and w.name in MEASURED_TRAFFIC:
         t_bytes, t_profile, t_src = MEASURED_TRAFFIC[w.name]
         if t_src == kernel_source_id():
             traffic, traffic_source = t_bytes, t_profile
@@ -134,6 +140,21 @@ def main():
         "launch_ms": [round(float(x), 4) for x in launch_ms.mean(axis=0)],
     }
     timed.close()
+
+    # ---- the other forward (steps kept apart unless --step-partials, which swaps the two)
+    other = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=w.graph, layout=args.layout,
+                              half_partials=w.half_partials, step_partials=not args.step_partials)
+    for _ in range(2):
+        other.forward(qd, kd, vd, out, lse, stream)
+    ev0.record(stream)
+    for _ in range(args.steps):
+        other.forward(qd, kd, vd, out, lse, stream)
+    ev1.record(stream)
+    torch.cuda.synchronize()
+    other_ms = ev0.elapsed_time(ev1) / args.steps
+    other_leg = {"ms_per_step_events": round(other_ms, 4), "tflops": round(w.flops / (other_ms * 1e-3) / 1e12, 2),
+                 "workspace_bytes": int(other.lib.ringattn_workspace_bytes(other.params))}
+    other.close()
 
     # ---- merge kernel alone: the ring merge on caller-held partials (random numbers: only the
     # bytes matter), events on the launch stream
@@ -217,6 +238,7 @@ def main():
                 "lockstep_ms": round(lockstep, 4),
                 "per_gpu_tflops_in_lockstep": round(w.flops / P / (lockstep * 1e-3) / 1e12, 1)}
     eager.close()
+    plan_ws = plan.lib.ringattn_workspace_bytes(plan.params)
     plan.close()
 
     # ---- CPU baseline: the oracle (a port; the reference has no CPU attention path) on a
@@ -247,9 +269,13 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "ms_per_step_events": round(ms_per_step_events, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w.dtype, "data": "synthetic",
         "config": {"workload": describe(w), "algorithmic_flop": w.flops, "graph": bool(w.graph), "layout": args.layout,
-                   "partials": "fp16" if w.half_partials else "fp32"},
+                   "partials": ("fp16" if w.half_partials else "fp32") if args.step_partials
+                   else "none: softmax state carried through the ring steps in registers",
+                   "workspace_bytes": int(plan_ws)},
         "pct_mfma_peak": round(100.0 * tflops / peak, 2),
-        "roofline": roofline, "merge": merge, "per_ring_step": per_step, "rank_local_ring": ring, "cpu_baseline": cpu,
+        "roofline": roofline,
+        ("forward_with_carried_state" if args.step_partials else "forward_with_step_partials"): other_leg,
+        "merge": merge, "per_ring_step": per_step, "rank_local_ring": ring, "cpu_baseline": cpu,
     }))
 
 

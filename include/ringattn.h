@@ -53,7 +53,14 @@ extern "C" {
 #define RINGATTN_FLAG_HALF_PARTIALS 4 /* keep the per-step partial O in fp16 instead of fp32 (for either input dtype): halves
                                       the workspace and the bytes the block kernel writes and the merge reads.  A partial O
                                       row is a weighted mean of V rows, so this needs |V| < 65504, and it adds up to 2^-11
-                                      relative error per partial (fp32 partials add none); the partial LSE stays fp32 */
+                                      relative error per partial (fp32 partials add none); the partial LSE stays fp32.
+                                      Applies wherever partials are written (ringattn_block_fwd, ringattn_rank_step_fwd,
+                                      ringattn_fwd with RINGATTN_FLAG_STEP_PARTIALS) */
+#define RINGATTN_FLAG_STEP_PARTIALS 8 /* ringattn_fwd keeps the ring steps apart: a normalised partial (O, LSE) per step in
+                                      the workspace, merged at the end -- the arithmetic of ringattn_block_fwd +
+                                      ringattn_merge_ring, bit for bit, in one launch.  Without the flag (the default)
+                                      the softmax state (max, sum, acc-O) runs through all steps in registers, as in the
+                                      reference's kernel (csrc/ring_attention.cu:439-443,597), and no workspace is needed */
 
 /*
  * Placement of the sequence on the ranks.  CONTIGUOUS: rank r holds the tokens that follow
@@ -94,16 +101,17 @@ typedef struct ringattn_params {
 
 typedef struct ringattn_plan ringattn_plan;
 
-/* Bytes of device workspace a plan needs: one partial O row and one partial LSE per query row
- * and VISIBLE ring step -- (dim + 1) * 4 bytes each, (2 dim + 4) with RINGATTN_FLAG_HALF_PARTIALS.
- * Without a mask every row has npes steps; with the causal mask a row of rank r has r + 1 (36 of
- * the 64 (rank, step) pairs at npes = 8); with the zigzag layout the low half of rank r has r + 1
- * and the high half npes.  0 if the parameters are invalid. */
+/* Bytes of device workspace a plan needs.  0 unless RINGATTN_FLAG_STEP_PARTIALS is set; then one
+ * partial O row and one partial LSE per query row and VISIBLE ring step -- (dim + 1) * 4 bytes
+ * each, (2 dim + 4) with RINGATTN_FLAG_HALF_PARTIALS.  Without a mask every row has npes steps;
+ * with the causal mask a row of rank r has r + 1 (36 of the 64 (rank, step) pairs at npes = 8);
+ * with the zigzag layout the low half of rank r has r + 1 and the high half npes.  Also 0 if the
+ * parameters are invalid. */
 size_t ringattn_workspace_bytes(const ringattn_params* params);
 
 /*
- * Create a plan: validates the parameters and allocates the workspace ONCE -- the
- * job set_params_fprop (csrc/ring_attention.cu:361-395) does on every call with a
+ * Create a plan: validates the parameters and allocates the workspace (if the plan needs one)
+ * ONCE -- the job set_params_fprop (csrc/ring_attention.cu:361-395) does on every call with a
  * cudaMalloc and two nvshmem_mallocs that are never freed (:383-394).
  * If workspace != NULL it is used instead of an internal allocation and must hold
  * at least ringattn_workspace_bytes() bytes (workspace_bytes is checked).
@@ -117,8 +125,10 @@ int ringattn_plan_destroy(ringattn_plan* plan);
 /*
  * The whole forward for all npes virtual ranks: replaces ring_attention()
  * (csrc/ring_attention.cu:706-722) run on every PE.  ONE block-attention launch: a workgroup
- * owns 128 query rows, walks every ring step of those rows like the reference's CTA
- * (:439-443,456), writes a partial (O, LSE) per step into the workspace and merges them.
+ * owns 128 query rows and walks every ring step of those rows with the running max, sum and
+ * acc-O in registers, like the reference's CTA (:439-443,456,597), then writes O = acc / sum
+ * (:621-664) and the LSE.  (With RINGATTN_FLAG_STEP_PARTIALS: a partial (O, LSE) per step into
+ * the workspace, merged at the end of the workgroup.)
  *   q, k, v : [batch, heads, S, dim] dtype     out : same shape and dtype
  *   lse     : [batch, heads, S] fp32, natural log (the reference never writes it)
  * Asynchronous on `stream` (a hipStream_t, or NULL for the default stream); the
@@ -182,7 +192,9 @@ int ringattn_rank_step_fwd(ringattn_plan* plan, int rank, int step, const void* 
  * The merge of one rank's per-step partials: o_parts [npes, batch*heads*h_seqlen[rank], dim] and
  * lse_parts [npes, batch*heads*h_seqlen[rank]], slot s as written by ringattn_rank_step_fwd for
  * step s (slots of steps that left the rows untouched are not read); out / lse hold the rank's
- * rows only.  Bit-identical to the rows ringattn_fwd produces for this rank.
+ * rows only.  Bit-identical to the rows ringattn_fwd produces for this rank on a plan with
+ * RINGATTN_FLAG_STEP_PARTIALS (without the flag ringattn_fwd rounds differently: it never
+ * normalises per step).
  */
 int ringattn_rank_merge(ringattn_plan* plan, int rank, const void* o_parts, const float* lse_parts, void* out,
                         float* lse, void* stream);
@@ -244,13 +256,13 @@ int ringattn_ring_attention(const void* q, const void* k, const void* v, void* o
  * reference (whose entry allocates on every call, csrc/ring_attention.cu:383-394).  Same
  * arguments and results as ringattn_ring_attention, plus the stream; it calls no hipMalloc,
  * hipFree, memcpy or other allocating routine and does not synchronise: the work (a
- * table-writing kernel, then the block kernel with its fused merge) is queued on `stream`.  The per-step
- * partials live in a static device array of ringattn_noalloc_scratch_bytes() bytes (32 MiB,
- * held by every GPU the library runs on until the process ends); a call that needs more --
- * visible_steps * (seqlen[mype] * (dim + 1) * 4 + 32) + seqlen[mype] * 4 + 64 bytes, visible_steps
- * being npes, or mype + 1 with the causal mask -- returns RINGATTN_ERR_WORKSPACE.  All calls on
- * one GPU share that array: calls that overlap on one GPU (two streams, two threads) race;
- * nothing in it needs clearing between calls.
+ * table-writing kernel, then the block kernel) is queued on `stream`.  The table of ring steps
+ * the block kernel reads (32 bytes + 32 per visible step), which ringattn_ring_attention keeps
+ * in a per-call allocation, lives in a static device array of ringattn_noalloc_scratch_bytes()
+ * bytes (4 KiB, held by every GPU the library runs on until the process ends): enough for
+ * RINGATTN_MAX_NPES steps, and a ring with more ranks is refused with RINGATTN_ERR_NPES like
+ * everywhere else.  All calls on one GPU share that array: calls that overlap on one GPU (two
+ * streams, two threads) race; nothing in it needs clearing between calls.
  */
 int ringattn_ring_attention_noalloc(const void* q, const void* k, const void* v, void* out, float* lse,
                                     int npes, int mype, const int* seqlen, int dim, int max_seq,

@@ -19,6 +19,7 @@ TORCH_DTYPE = {0: torch.float16, 1: torch.bfloat16}
 FLAG_GRAPH = 1
 FLAG_TIMING = 2
 FLAG_HALF_PARTIALS = 4
+FLAG_STEP_PARTIALS = 8
 LAYOUT_CODE = {"contiguous": 0, "zigzag": 1}
 
 
@@ -74,14 +75,18 @@ class RingAttention:
     """A forward plan for P virtual ring ranks on one GPU."""
 
     def __init__(self, npes, chunk, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, graph=False,
-                 kv_heads=0, layout="contiguous", timing=False, half_partials=False, workspace=None):
+                 kv_heads=0, layout="contiguous", timing=False, half_partials=False, workspace=None,
+                 step_partials=False):
         """`chunk`: tokens per rank -- one int for equal chunks or a list of npes lengths
         (the per-PE seqlen[] of csrc/ring_attention.cu:753).  `kv_heads`: heads of K and V for
         grouped-query attention (0 = same as `heads`).  `layout`: "contiguous" (rank r holds
         the tokens after those of rank r-1) or "zigzag" (rank r holds a low and a high
-        half-chunk; see zigzag_order).  `half_partials`: keep the per-step partial O in fp16
-        (half the workspace and merge traffic; needs |V| < 65504).  `workspace`: a (device address,
-        bytes) pair the caller owns and keeps alive, instead of an allocation by the plan."""
+        half-chunk; see zigzag_order).  `step_partials`: forward() keeps the ring steps apart (a
+        partial (O, LSE) per step in the workspace, merged at the end: the arithmetic of
+        block_forward + merge_ring) instead of carrying the softmax state through all steps in
+        registers.  `half_partials`: keep per-step partial O in fp16 (half the workspace and merge
+        traffic; needs |V| < 65504).  `workspace`: a (device address, bytes) pair the caller owns
+        and keeps alive, instead of an allocation by the plan (only a step_partials plan needs one)."""
         self.lib = _lib.load()
         self.seqlen = [int(chunk)] * npes if isinstance(chunk, int) else [int(x) for x in chunk]
         if len(self.seqlen) != npes:
@@ -95,7 +100,8 @@ class RingAttention:
         self.kv_heads = kv_heads if kv_heads else heads
         self.params = make_params(npes, self.seqlen, dim, batch, heads, dtype, causal, softmax_scale,
                                   (FLAG_GRAPH if graph else 0) | (FLAG_TIMING if timing else 0)
-                                  | (FLAG_HALF_PARTIALS if half_partials else 0), kv_heads,
+                                  | (FLAG_HALF_PARTIALS if half_partials else 0)
+                                  | (FLAG_STEP_PARTIALS if step_partials else 0), kv_heads,
                                   LAYOUT_CODE[layout])
         self.handle = ctypes.c_void_p()
         ws_ptr, ws_bytes = (None, 0) if workspace is None else (ctypes.c_void_p(int(workspace[0])), int(workspace[1]))

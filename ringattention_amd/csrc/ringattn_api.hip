@@ -91,6 +91,7 @@ int validate(const ringattn_params* p, Derived* d) {
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 inline bool half_partials(const ringattn_params& p) { return (p.flags & RINGATTN_FLAG_HALF_PARTIALS) != 0; }
+inline bool step_partials(const ringattn_params& p) { return (p.flags & RINGATTN_FLAG_STEP_PARTIALS) != 0; }
 
 inline ringattn::WorkItem make_item(int q_start, int q_len, int kv_start, int kv_len, int diag_off, int slot) {
   ringattn::WorkItem w;
@@ -181,9 +182,10 @@ std::vector<HostSegment> forward_segments(const Derived& d, int P, bool causal) 
   return segs;
 }
 
-// Workspace of a forward: one partial block [batch*heads, len] rows per (segment, item) --
-// only the (rank, step) pairs the mask leaves visible -- partial O of every block first (fp32,
-// or fp16 with RINGATTN_FLAG_HALF_PARTIALS), then the fp32 partial LSEs.
+// Workspace of a forward that keeps per-step partials (RINGATTN_FLAG_STEP_PARTIALS; none
+// otherwise): one partial block [batch*heads, len] rows per (segment, item) -- only the
+// (rank, step) pairs the mask leaves visible -- partial O of every block first (fp32, or fp16
+// with RINGATTN_FLAG_HALF_PARTIALS), then the fp32 partial LSEs.
 int64_t partial_rows_of(const std::vector<HostSegment>& segs, const Derived& d) {
   int64_t rows = 0;
   for (const auto& sg : segs) rows += (int64_t)sg.items.size() * d.BH * sg.len;
@@ -191,6 +193,7 @@ int64_t partial_rows_of(const std::vector<HostSegment>& segs, const Derived& d) 
 }
 
 size_t workspace_bytes_of(const ringattn_params* p, const Derived& d) {
+  if (!step_partials(*p)) return 0;
   const size_t o_elem = half_partials(*p) ? 2 : 4;
   const int64_t rows = partial_rows_of(forward_segments(d, p->npes, p->causal != 0), d);
   return (size_t)rows * ((size_t)p->dim * o_elem + sizeof(float));
@@ -431,9 +434,10 @@ int launch_slice(const ringattn_plan* pl, const TableSlice& sl, ringattn::BlockA
   return RINGATTN_OK;
 }
 
-// The ring step loop (csrc/ring_attention.cu:456-620) plus the merge, ONE launch: every
-// workgroup walks the ring steps of its 128 rows, writes a partial (O, LSE) per step and
-// merges them at the end.
+// The ring step loop (csrc/ring_attention.cu:456-620) and the epilogue (:621-664), ONE launch:
+// every workgroup walks the ring steps of its 128 rows with the softmax state carried in
+// registers, like the reference's CTA (:439-443,597).  With RINGATTN_FLAG_STEP_PARTIALS it
+// writes a partial (O, LSE) per step instead and merges them at the end.
 int run_forward(ringattn_plan* pl, const void* q, const void* k, const void* v, void* out,
                 float* lse, hipStream_t stream) {
   const bool timing = (pl->p.flags & RINGATTN_FLAG_TIMING) && !(pl->p.flags & RINGATTN_FLAG_GRAPH);
@@ -446,7 +450,7 @@ int run_forward(ringattn_plan* pl, const void* q, const void* k, const void* v, 
   a.lse_part = pl->lse_parts;
   a.out = out;
   a.lse = lse;
-  a.fuse_merge = 1;
+  a.mode = step_partials(pl->p) ? ringattn::kBlockPartialsMerged : ringattn::kBlockCarryState;
   a.groups = pl->d_groups;
   a.groups_per_xcd = pl->fwd_groups_per_xcd;
   if (timing) RA_HIP(hipEventRecord(pl->ev_t0, stream));
@@ -474,15 +478,14 @@ inline bool plan_ok(const ringattn_plan* pl) {
 
 // ---- the reference-shaped call for one rank (ringattn_ring_attention and its variant that
 // allocates nothing) ------------------------------------------------------------------------
-// Device scratch of one call: the rank's per-step partial O [n_parts, c, dim] fp32, partial LSE
-// [n_parts, c], a spare LSE row [c] for callers that pass no lse, and the segment + item table.
+// Device scratch of one call: the segment + item table the block kernel reads (the softmax state
+// is carried in registers across the ring steps, so there are no partials to park).
 struct RankCall {
   ringattn_params p;
   Derived d;
-  ringattn::TablePack pack;  // the visible ring steps of the rank in ring order, one compact slot each
+  ringattn::TablePack pack;  // the visible ring steps of the rank in ring order
   int n_parts = 0;
   int c = 0;                // rows of this rank
-  size_t lse_floats = 0;    // floats of the two LSE areas, padded so the table stays 32-byte aligned
   size_t scratch_bytes = 0;
 };
 
@@ -532,22 +535,17 @@ int prepare_rank_call(RankCall* rc, const void* q, const void* k, const void* v,
   }
   sg.item_count = rc->n_parts;
   if (rc->n_parts == 1) sg.last_item = -1;
-  rc->lse_floats = ((size_t)(rc->n_parts + 1) * c + 7) & ~(size_t)7;
-  rc->scratch_bytes = ((size_t)rc->n_parts * c * dim + rc->lse_floats) * sizeof(float) + sizeof(ringattn::Segment) +
-                      (size_t)rc->n_parts * sizeof(ringattn::SegItem);
+  rc->scratch_bytes = sizeof(ringattn::Segment) + (size_t)rc->n_parts * sizeof(ringattn::SegItem);
   return RINGATTN_OK;
 }
 
-// The table (written by a kernel from its arguments), then the block kernel with its fused
-// merge: two launches on `stream`, nothing is allocated or copied from the host.
-// `scratch`: rc.scratch_bytes of device memory.
+// The table (written by a kernel from its arguments), then the block kernel: two launches on
+// `stream`, nothing is allocated or copied from the host.
+// `scratch`: rc.scratch_bytes of device memory, 32-byte aligned.
 int run_rank_call(const RankCall& rc, void* scratch, const void* q, const void* k, const void* v, void* out,
                   float* lse, hipStream_t stream) {
   const int dim = rc.p.dim, c = rc.c, n_parts = rc.n_parts;
-  float* o_parts = (float*)scratch;
-  float* lse_parts = o_parts + (size_t)n_parts * c * dim;
-  float* lse_tmp = lse_parts + (size_t)n_parts * c;
-  ringattn::Segment* d_seg = (ringattn::Segment*)(lse_parts + rc.lse_floats);
+  ringattn::Segment* d_seg = (ringattn::Segment*)scratch;
   ringattn::SegItem* d_items = (ringattn::SegItem*)(d_seg + 1);
   RA_HIP(ringattn::launch_write_table(rc.pack, n_parts, d_seg, d_items, stream));
   ringattn::BlockArgs a;
@@ -555,11 +553,9 @@ int run_rank_call(const RankCall& rc, void* scratch, const void* q, const void* 
   a.q = q;
   a.k = k;
   a.v = v;
-  a.o_part = o_parts;
-  a.lse_part = lse_parts;
   a.out = out;
-  a.lse = lse ? lse : lse_tmp;
-  a.fuse_merge = 1;
+  a.lse = lse;  // may be NULL
+  a.mode = ringattn::kBlockCarryState;
   a.segs = d_seg;
   a.items = d_items;
   a.n_segs = 1;
@@ -573,7 +569,9 @@ int run_rank_call(const RankCall& rc, void* scratch, const void* q, const void* 
 // Static device scratch of ringattn_ring_attention_noalloc.  In host code the array's name is
 // only a handle for hipGetSymbolAddress; the device address is looked up once per device
 // (each GPU holds its own copy of the array) and kept.
-constexpr size_t kScratchBytes = (size_t)32 << 20;
+constexpr size_t kScratchBytes = 4096;
+static_assert(kScratchBytes >= sizeof(ringattn::Segment) + RINGATTN_MAX_NPES * sizeof(ringattn::SegItem),
+              "the table of the largest ring fits");
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mu;
@@ -646,7 +644,7 @@ int ringattn_plan_create(const ringattn_params* params, void* workspace, size_t 
   if (workspace) {
     pl->ws = workspace;
     pl->own_ws = false;
-  } else {
+  } else if (need > 0) {
     hipError_t e = hipMalloc(&pl->ws, need);
     if (e != hipSuccess) {
       delete pl;

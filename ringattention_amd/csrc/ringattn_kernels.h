@@ -52,14 +52,23 @@ struct Segment {
 };
 static_assert(sizeof(Segment) == 32, "Segment is read as two 16-byte scalar loads");
 
+// What a workgroup of the block kernel does with the softmax state (max, sum, acc-O) of its rows
+// between the KV chunks it walks.
+enum BlockMode {
+  kBlockPartials = 0,        // per chunk: emit the normalised partial (O, LSE), reset the state
+  kBlockPartialsMerged = 1,  // the same, and after the last chunk merge the partials of the rows into out / lse
+  kBlockCarryState = 2,      // carry the state across the chunks, as the reference's CTA does across its ring
+                             // steps (csrc/ring_attention.cu:439-443,597), and write out / lse once: no partials
+};
+
 struct BlockArgs {
   const void* q;       // [BH, S, D] storage dtype
   const void* k;       // [batch * heads / kv_group, S, D]
   const void* v;       // [batch * heads / kv_group, S, D]
   void* o_part;        // partial O rows (normalised), fp32 or fp16 (half_partials); indexed by SegItem::part_base
-  float* lse_part;     // partial LSE rows (natural log), same row numbering
-  void* out;           // fuse_merge: [BH, S, D] storage dtype
-  float* lse;          // fuse_merge: [BH, S]
+  float* lse_part;     // partial LSE rows (natural log), same row numbering; both unused with kBlockCarryState
+  void* out;           // unless kBlockPartials: [BH, S, D] storage dtype
+  float* lse;          // unless kBlockPartials: [BH, S]; may be NULL with kBlockCarryState
   const Segment* segs; // device arrays
   const SegItem* items;
   const int2* groups;  // NULL, or [8][groups_per_xcd] (segment, head) pairs: what the workgroups of each XCD run,
@@ -75,7 +84,7 @@ struct BlockArgs {
   int kv_group;        // query heads per KV head (1 = one KV head per query head)
   float scale_log2;    // softmax_scale * log2(e)
   int half_partials;   // partial O stored as fp16 instead of fp32
-  int fuse_merge;      // after its last item a workgroup merges the partials of its rows into out / lse
+  int mode;            // BlockMode
 };
 
 // Merge of (O, LSE) partials into the final O (storage dtype) and LSE, for row ranges of every

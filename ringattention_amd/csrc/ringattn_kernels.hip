@@ -42,6 +42,7 @@ namespace ringattn {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -67,6 +68,7 @@ template <int DT> struct Elem;
 template <> struct Elem<0> {
   using type = _Float16;
   using vec8 = f16x8;
+  using vec4 = f16x4;
   static __device__ __forceinline__ f32x16 mma(s16x8 a, s16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(vec8, a), __builtin_bit_cast(vec8, b), c, 0, 0, 0);
   }
@@ -74,6 +76,7 @@ template <> struct Elem<0> {
 template <> struct Elem<1> {
   using type = __bf16;
   using vec8 = bf16x8;
+  using vec4 = bf16x4;
   static __device__ __forceinline__ f32x16 mma(s16x8 a, s16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(vec8, a), __builtin_bit_cast(vec8, b), c, 0, 0, 0);
   }
@@ -779,11 +782,37 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockArgs
     }
   };
 
+  // the rows' final result from a state carried over every chunk: the reference's epilogue
+  // (csrc/ring_attention.cu:621-664), O = acc / l in the storage type, plus the LSE
+  auto emit_result = [&]() {
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      const float l = cross_half_sum((ls[qb][0] + ls[qb][1]) + (ls[qb][2] + ls[qb][3]));
+      const float inv = (l > 0.f) ? 1.f / l : 0.f;
+      const int row_l = qt * BM + 32 * QB * wave + 32 * qb + n;
+      if (row_l >= q_len) continue;  // a row beyond the query range
+      const int64_t row = (int64_t)bh * a.S + q_start + row_l;
+      typename E::type* orow = (typename E::type*)a.out + row * D;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          typename E::vec4 val;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) val[e] = (typename E::type)(oacc[qb][db][4 * q4 + e] * inv);
+          *(typename E::vec4*)(orow + 32 * db + 8 * q4 + 4 * h) = val;
+        }
+      if (h == 0 && a.lse) a.lse[row] = (l > 0.f) ? (ms[qb] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
+    }
+  };
+
   using C0 = std::integral_constant<int, 0>;
   using C1 = std::integral_constant<int, 1>;
   using C2 = std::integral_constant<int, 2>;
   using C3 = std::integral_constant<int, 3>;
 
+  const bool keep_state = a.mode == kBlockCarryState;
+  bool fresh = true;     // the softmax state is empty: the chunk's first tile sets the reference max
   bool carried = false;  // the previous chunk's pipeline ran on into this one
   for (int it = 0; it < n_items; ++it) {
     const SegItem* w = item_at(it);
@@ -825,7 +854,8 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockArgs
       float cand[QB];
       mask_tile(s_even, 0, kUnchecked);
       tile_maxes(s_even, cand);
-      set_reference(cand);
+      if (fresh) set_reference(cand);
+      else move_reference(cand, true);
     }
 
     // Steady blocks come in groups of four (ring slots are compile-time constants).  A group
@@ -856,19 +886,29 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockArgs
       if (u & 1) block(C1{}, std::false_type{}, std::false_type{}, u);
       else block(C0{}, std::false_type{}, std::false_type{}, u);
     }
+    carried = carry;
+    if (keep_state) {
+      // the softmax state runs on into the next chunk; with the pipeline carried over as well,
+      // the chunk boundary is just another tile boundary
+      fresh = false;
+      if (!carry) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // re-reads of the last tile
+      continue;
+    }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next chunk's first tiles, or re-reads of the last tile
     if (carry) {
       __syncthreads();
       synced = true;
     }
-
     emit_partial(w);
     reset_state();
-    carried = carry;
+  }
+  if (keep_state) {
+    emit_result();
+    return;
   }
 
   // ---- fused merge: this workgroup's rows over the partials it has just written
-  if (a.fuse_merge) {
+  if (a.mode == kBlockPartialsMerged) {
     static_assert(sizeof(smem) >= kMaxParts * BM * sizeof(float), "partial LSEs of a q tile fit the rings");
     merge_job_rows<DT, D, HP>(a.o_part, a.lse_part, a.out, a.lse, a.items, seg, bh, qt, a.S,
                               (lds_float*)(__attribute__((address_space(3))) void*)smem);

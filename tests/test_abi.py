@@ -12,6 +12,7 @@ from ringattention_amd._lib import RingattnParams
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 OK, E_NULL, E_NPES, E_DIM, E_DTYPE, E_SEQLEN, E_SHAPE, E_WS, E_RANK, E_PLAN, E_HIP, E_ALLOC, E_ALIGN = range(13)
+STEP_PARTIALS = 8   # RINGATTN_FLAG_STEP_PARTIALS
 
 
 def params(npes=2, seqlen=(128, 128), dim=64, batch=1, heads=1, dtype=0, causal=0, flags=0, scale=0.0, kv_heads=0, layout=0):
@@ -45,8 +46,9 @@ def test_header_constants_match_error_strings(ralib):
 
 def test_parameter_validation(ralib):
     wb = ralib.ringattn_workspace_bytes
-    assert wb(ctypes.byref(params())) == 2 * 256 * 65 * 4
-    assert wb(ctypes.byref(params(seqlen=(128, 384)))) == 2 * 512 * 65 * 4   # unequal per-rank lengths are fine
+    assert wb(ctypes.byref(params())) == 0          # the softmax state is carried in registers: no partials to park
+    assert wb(ctypes.byref(params(flags=STEP_PARTIALS))) == 2 * 256 * 65 * 4
+    assert wb(ctypes.byref(params(seqlen=(128, 384), flags=STEP_PARTIALS))) == 2 * 512 * 65 * 4   # unequal per-rank lengths are fine
     h = ctypes.c_void_p()
 
     def create(p):
@@ -64,8 +66,8 @@ def test_parameter_validation(ralib):
         assert create(params(dim=bad_dim)) == E_DIM
     assert create(params(dtype=2)) == E_DTYPE
     assert create(params(dtype=-1)) == E_DTYPE
-    assert wb(ctypes.byref(params(seqlen=(128, 200)))) == 2 * 328 * 65 * 4   # nor need they be multiples of the tile
-    assert wb(ctypes.byref(params(seqlen=(1, 3)))) == 2 * 4 * 65 * 4
+    assert wb(ctypes.byref(params(seqlen=(128, 200), flags=STEP_PARTIALS))) == 2 * 328 * 65 * 4   # nor need they be multiples of the tile
+    assert wb(ctypes.byref(params(seqlen=(1, 3), flags=STEP_PARTIALS))) == 2 * 4 * 65 * 4
     assert create(params(seqlen=(0, 128))) == E_SEQLEN
     assert create(params(seqlen=(0, 0))) == E_SEQLEN
     assert create(params(seqlen=(-128, -128))) == E_SEQLEN
@@ -82,28 +84,30 @@ def test_parameter_validation(ralib):
 
 
 def test_workspace_counts_only_visible_steps(ralib):
-    # one partial row per query row and VISIBLE ring step: causal ranks hold r + 1 steps, not npes
+    # a plan that keeps the ring steps apart: one partial row per query row and VISIBLE ring step
+    # (causal ranks hold r + 1 steps, not npes)
     wb = ralib.ringattn_workspace_bytes
     row = (128 + 1) * 4
-    dense = wb(ctypes.byref(params(npes=8, seqlen=(4096,) * 8, dim=128, heads=32, causal=0)))
-    causal = wb(ctypes.byref(params(npes=8, seqlen=(4096,) * 8, dim=128, heads=32, causal=1)))
+    assert wb(ctypes.byref(params(npes=8, seqlen=(4096,) * 8, dim=128, heads=32, causal=1))) == 0
+    dense = wb(ctypes.byref(params(npes=8, seqlen=(4096,) * 8, dim=128, heads=32, causal=0, flags=STEP_PARTIALS)))
+    causal = wb(ctypes.byref(params(npes=8, seqlen=(4096,) * 8, dim=128, heads=32, causal=1, flags=STEP_PARTIALS)))
     assert dense == 8 * 32 * 32768 * row
     assert causal == 36 * 32 * 4096 * row and causal * 64 == dense * 36       # 36 of the 64 (rank, step) pairs
     # zigzag: the low half of rank r sees r + 1 steps, the high half all 8: (36 + 64) / 2 of 64 chunk-steps
-    zig = wb(ctypes.byref(params(npes=8, seqlen=(4096,) * 8, dim=128, heads=32, causal=1, layout=1)))
+    zig = wb(ctypes.byref(params(npes=8, seqlen=(4096,) * 8, dim=128, heads=32, causal=1, layout=1, flags=STEP_PARTIALS)))
     assert zig == (36 + 64) * 32 * 2048 * row
     # fp16 partials (flag 4): 2 dim + 4 bytes per partial row
-    half = wb(ctypes.byref(params(npes=8, seqlen=(4096,) * 8, dim=128, heads=32, causal=1, flags=4)))
+    half = wb(ctypes.byref(params(npes=8, seqlen=(4096,) * 8, dim=128, heads=32, causal=1, flags=4 | STEP_PARTIALS)))
     assert half == 36 * 32 * 4096 * (2 * 128 + 4)
     # ragged, unequal ranks
     lens = (100, 333, 1, 77)
-    ragged = wb(ctypes.byref(params(npes=4, seqlen=lens, dim=64, causal=1)))
+    ragged = wb(ctypes.byref(params(npes=4, seqlen=lens, dim=64, causal=1, flags=STEP_PARTIALS)))
     assert ragged == sum((r + 1) * n for r, n in enumerate(lens)) * (64 + 1) * 4
 
 
 def test_plan_lifetime_with_caller_workspace(ralib):
     # a caller-provided workspace needs no HIP call, so the plan life cycle runs on a CPU host
-    p = params()
+    p = params(flags=STEP_PARTIALS)
     need = ralib.ringattn_workspace_bytes(ctypes.byref(p))
     ws = np.zeros(need // 4 + 8, dtype=np.float32)
     base = ws.ctypes.data + (-ws.ctypes.data % 16)
@@ -165,10 +169,10 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
 
 
 def _plan_on_host(ralib, p):
-    # the workspace of a plan is never touched on the host: any aligned address will do
-    need = ralib.ringattn_workspace_bytes(ctypes.byref(p))
+    # a plan that carries the softmax state needs no workspace, so creating it makes no HIP call
+    assert ralib.ringattn_workspace_bytes(ctypes.byref(p)) == 0
     h = ctypes.c_void_p()
-    assert ralib.ringattn_plan_create(ctypes.byref(p), ctypes.c_void_p(1 << 20), need, ctypes.byref(h)) == OK
+    assert ralib.ringattn_plan_create(ctypes.byref(p), None, 0, ctypes.byref(h)) == OK
     return h
 
 
@@ -297,8 +301,7 @@ def test_python_front_end_refuses_wrongly_shaped_tensors(ralib):
     import torch
     from ringattention_amd import api
     P, c, d, B, H = 4, 128, 64, 2, 3
-    need = ralib.ringattn_workspace_bytes(ctypes.byref(params(npes=P, seqlen=(c,) * P, dim=d, batch=B, heads=H)))
-    plan = api.RingAttention(P, c, d, B, H, "fp16", False, workspace=(1 << 20, need))   # host only: never launched
+    plan = api.RingAttention(P, c, d, B, H, "fp16", False)   # needs no workspace; host only: never launched
     S = P * c
     good = torch.zeros(B, H, S, d, dtype=torch.float16)
     with pytest.raises(ValueError, match="k must have shape"):

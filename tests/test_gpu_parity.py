@@ -63,7 +63,11 @@ def check_rows(oracle, w, q, k, v, out, lse, rows, scale=None, half_partials=Non
     storage type where that is more (a bf16 value in [4, 8) is a multiple of 2^-5, so even the correctly
     rounded result can be 1.56e-2 off; only the first rows of a causal sequence, which average very few
     V rows, get that large) -- and within ONE unit in the last place (of the row's largest element) of the
-    oracle rounded to the storage type (two with fp16 per-step partials).  LSE: relative error <= 1e-3."""
+    oracle rounded to the storage type (two with fp16 per-step partials), or, where that is more, within
+    what rounding the probabilities to the storage type allows (each p is off by at most half an ulp
+    relative and O is a p-weighted mean of V rows: 2^-(mantissa+1) max|V|) plus half an ulp for the store;
+    only rows whose few dominant keys carry large V entries that nearly cancel reach the second form.
+    LSE: relative error <= 1e-3."""
     o_ref, l_ref = oracle.attention_rows(q, k, v, w.dtype, causal=w.causal, rows=rows, scale=scale)
     idx = torch.from_numpy(rows).cuda()
     o_gpu = out.reshape(-1, w.dim)[idx].double().cpu().numpy()
@@ -88,7 +92,15 @@ def check_rows(oracle, w, q, k, v, out, lse, rows, scale=None, half_partials=Non
     assert (err <= tol).all(), f"{w.name}: max|dO| = {err_o:.3e}, worst excess {(err - tol).max():.3e}"
     # fp16 per-step partials (RINGATTN_FLAG_HALF_PARTIALS) round once more on the way: two units then
     ulps = 2 if (w.half_partials if half_partials is None else half_partials) else 1
-    assert (err_r <= ulps * ulp_r).all(), f"{w.name}: {(err_r / ulp_r).max():.2f} ulp from the rounded oracle"
+    v_max = bits_to_float64(np.array([(np.ascontiguousarray(v).view(np.uint16) & 0x7FFF).max()], dtype=np.uint16), w.dtype)[0]
+    p_rounding = 2.0 ** -((10 if w.dtype == "fp16" else 7) + 1) * v_max + 0.5 * storage_ulp(o_rounded, w.dtype)
+    over = int((err_r > ulps * ulp_r).any(axis=1).sum())
+    if over:
+        print(f"parity {w.name}: {over} of {len(rows)} rows beyond {ulps} ulp of the rounded oracle "
+              f"(max {(err_r / ulp_r).max():.2f}), within the p-rounding bound {p_rounding.max():.3e}")
+    assert over <= max(1, len(rows) // 1000), f"{w.name}: {over} rows beyond {ulps} ulp of the rounded oracle"
+    assert (err_r <= np.maximum(ulps * ulp_r, p_rounding)).all(), \
+        f"{w.name}: {(err_r / ulp_r).max():.2f} ulp from the rounded oracle, beyond the p-rounding bound"
     assert err_l <= LSE_RTOL, f"{w.name}: max rel dLSE = {err_l:.3e}"
     return err_o, err_l
 
@@ -140,12 +152,15 @@ def test_causal_small_golden(oracle):
     assert np.abs(out.float().cpu().numpy() - g["o_f32"]).max() <= O_TOL
 
 
-@pytest.mark.parametrize("name", ["cfg2", "cfg3", "cfg4", "cfg5"])
-def test_workload_whole_heads(oracle, name):
+@pytest.mark.parametrize("name,step_partials", [("cfg2", False), ("cfg2", True), ("cfg3", False), ("cfg3", True),
+                                                ("cfg4", False), ("cfg4", True), ("cfg5", False)])
+def test_workload_whole_heads(oracle, name, step_partials):
+    # step_partials: the forward that keeps the ring steps apart (per-step partials in the workspace,
+    # fp16 where the workload says so) instead of carrying the softmax state through them
     w = WORKLOADS[name]
     q, k, v = api.make_qkv_bits(w)
-    out, lse = forward(w, q, k, v)
-    check_rows(oracle, w, q, k, v, out, lse, workload_rows(w))
+    out, lse = forward(w, q, k, v, step_partials=step_partials)
+    check_rows(oracle, w, q, k, v, out, lse, workload_rows(w), half_partials=w.half_partials and step_partials)
     # full-size properties: finite everywhere, convexity |O| <= max|V| (O is an average of V rows)
     assert torch.isfinite(out).all() and torch.isfinite(lse).all()
     vmax = np.abs(bits_to_float64(v, w.dtype)).max()
@@ -302,7 +317,13 @@ def test_zigzag_layout(oracle, seqlen, B, H, d, dtype, hkv):
     out_seq, lse_seq = out[:, :, inv].contiguous(), lse[:, :, inv].contiguous()
     k_full, v_full = ((np.repeat(x, H // hkv, axis=1) if hkv else x) for x in (k, v))
     check_rows(oracle, w, q, k_full, v_full, out_seq, lse_seq, np.arange(w.rows))
-    # step by step through the C ABI: the same items, so the same bits
+    plan.close()
+    # the forward that keeps the steps apart: same bar against the oracle ...
+    plan = api.RingAttention(P, list(seqlen), d, B, H, dtype, True, kv_heads=hkv, layout="zigzag", step_partials=True)
+    out, lse = plan.forward(qd, kd, vd)
+    torch.cuda.synchronize()
+    check_rows(oracle, w, q, k_full, v_full, out[:, :, inv].contiguous(), lse[:, :, inv].contiguous(), np.arange(w.rows))
+    # ... and step by step through the C ABI: the same items, so the same bits
     o_parts = torch.zeros((P, B, H, S, d), dtype=torch.float32, device="cuda")
     lse_parts = torch.full((P, B, H, S), float("-inf"), dtype=torch.float32, device="cuda")
     for s in range(P):
@@ -543,7 +564,9 @@ def test_random_plans_against_oracle(oracle):
         H, S = hkv * group, sum(lens)
         scale = float(rng.choice([0.0, 0.05, 0.2]))
         graph = bool(rng.integers(0, 2))
-        tag = f"case {case}: P={P} lens={lens} B={B} H={H} hkv={hkv} d={d} {dtype} causal={causal} zigzag={zigzag} scale={scale} graph={graph}"
+        steps_apart = case % 3 == 2
+        tag = (f"case {case}: P={P} lens={lens} B={B} H={H} hkv={hkv} d={d} {dtype} causal={causal} zigzag={zigzag} "
+               f"scale={scale} graph={graph} step_partials={steps_apart}")
         print(tag, flush=True)
         w = Workload("rand", B, H, d, 1, S, dtype, 1000 + case, causal)
         q, _, _ = api.make_qkv_bits(w)
@@ -552,7 +575,8 @@ def test_random_plans_against_oracle(oracle):
         inv = torch.from_numpy(np.argsort(order)).cuda()
         qd, kd, vd = (to_dev(np.ascontiguousarray(x[:, :, order]), dtype) for x in (q, k, v))
         plan = api.RingAttention(P, lens, d, B, H, dtype, causal, softmax_scale=scale, graph=graph,
-                                 kv_heads=hkv if group > 1 else 0, layout="zigzag" if zigzag else "contiguous")
+                                 kv_heads=hkv if group > 1 else 0, layout="zigzag" if zigzag else "contiguous",
+                                 step_partials=steps_apart)
         out, lse = plan.forward(qd, kd, vd)
         if graph:                                   # a replay of the captured graph must give the same bits
             out2, lse2 = plan.forward(qd, kd, vd, torch.empty_like(out), torch.empty_like(lse))
@@ -606,8 +630,9 @@ def test_half_precision_partials(oracle, w, layout):
     order = api.zigzag_order([w.chunk] * w.npes) if layout == "zigzag" else np.arange(w.seq)
     inv = torch.from_numpy(np.argsort(order)).cuda()
     qd, kd, vd = (to_dev(np.ascontiguousarray(x[:, :, order]), w.dtype) for x in (q, k, v))
-    full = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, layout=layout)
-    half = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, layout=layout, half_partials=True)
+    full = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, layout=layout, step_partials=True)
+    half = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, layout=layout, step_partials=True,
+                             half_partials=True)
     wb = half.lib.ringattn_workspace_bytes
     assert wb(half.params) * (4 * w.dim + 4) == wb(full.params) * (2 * w.dim + 4)
     o32, l32 = full.forward(qd, kd, vd)
@@ -649,15 +674,26 @@ def test_half_precision_partials(oracle, w, layout):
 def test_rank_local_ring_equals_the_all_rank_forward(seqlen, causal, layout, d, dtype, hkv, half):
     # A ring of one process per GPU, replayed rank by rank on this GPU: every rank holds only its
     # own Q rows and, at step s, the K/V chunk of rank (r + s) mod P in a buffer of its own (what
-    # the exchange would have delivered).  Same work items, so the same bits as ringattn_fwd.
+    # the exchange would have delivered).  Same work items, so the same bits as a ringattn_fwd that
+    # keeps the steps apart; the default forward (state carried in registers) agrees to rounding.
     P, S, B, H = len(seqlen), sum(seqlen), 2, 4
     w = Workload("rank_local", B, H, d, 1, S, dtype, 111, causal)
     q, _, _ = api.make_qkv_bits(w)
     _, k, v = api.make_qkv_bits(Workload("rank_local_kv", B, hkv or H, d, 1, S, dtype, 112, causal))
     qd, kd, vd = (to_dev(x, dtype) for x in (q, k, v))
-    plan = api.RingAttention(P, list(seqlen), d, B, H, dtype, causal, kv_heads=hkv, layout=layout, half_partials=half)
+    plan = api.RingAttention(P, list(seqlen), d, B, H, dtype, causal, kv_heads=hkv, layout=layout, half_partials=half,
+                             step_partials=True)
     out, lse = plan.forward(qd, kd, vd)
+    carried = api.RingAttention(P, list(seqlen), d, B, H, dtype, causal, kv_heads=hkv, layout=layout)
+    out_c, lse_c = carried.forward(qd, kd, vd)
     torch.cuda.synchronize()
+    carried.close()
+    # per row: within two storage ulps of the row's largest element (three with fp16 partials)
+    ulp = 2.0**-10 if dtype == "fp16" else 2.0**-7
+    row_max = out.float().abs().amax(-1, keepdim=True)
+    exp2 = torch.exp2(torch.floor(torch.log2(row_max.clamp_min(2.0**-14))))
+    assert ((out_c.float() - out.float()).abs() <= (3 if half else 2) * ulp * exp2).all()
+    assert torch.allclose(lse_c, lse, rtol=1e-5, atol=1e-5)
     start = np.concatenate([[0], np.cumsum(seqlen)])
     for r in range(P):
         rows = slice(start[r], start[r + 1])

@@ -1,6 +1,6 @@
-"""The reference-shaped entry point that allocates nothing (static device scratch) against the
-allocating one, through the C ABI: same bits, on two calls in a row, the second on a smaller
-input (the scratch keeps the first call's contents)."""
+"""The reference-shaped entry point that allocates nothing (its table of ring steps lives in a
+static device scratch) against the allocating one, through the C ABI: same bits, on two calls
+in a row, the second on a smaller input (the scratch keeps the first call's contents)."""
 import numpy as np
 import pytest
 import torch
@@ -52,13 +52,16 @@ def test_noalloc_entry_without_lse_and_on_a_side_stream():
     assert torch.equal(out_a.view(torch.int16), out_b.view(torch.int16))
 
 
-def test_noalloc_entry_rejects_what_does_not_fit():
+def test_noalloc_entry_limits():
     lib = _lib.load()
-    cap = lib.ringattn_noalloc_scratch_bytes()
-    assert cap == 32 << 20
-    npes, c, dim = 8, 16384, 128          # 8 * 16384 * 129 * 4 bytes = 67.6 MB of partials
+    assert lib.ringattn_noalloc_scratch_bytes() == 4096
+    # the scratch holds the table of ring steps: 32 bytes + 32 per visible step, so 64 ranks fit ...
+    _run_pair(64, [64] * 64, 64, torch.float16, False, 17, seed=104)
+    _run_pair(8, [4096] * 8, 128, torch.bfloat16, True, 7, seed=105)      # ... whatever the lengths
+    # ... and a longer ring is refused as everywhere else
+    npes, c, dim = 65, 32, 64
     q = torch.zeros(c, dim, dtype=torch.float16, device="cuda")
     kv = torch.zeros(npes * c, dim, dtype=torch.float16, device="cuda")
     with pytest.raises(_lib.RingattnError) as e:
         api.ring_attention_noalloc(q, kv, kv, torch.empty_like(q), npes, 0, [c] * npes, dim, c)
-    assert e.value.code == 7              # RINGATTN_ERR_WORKSPACE
+    assert e.value.code == 2              # RINGATTN_ERR_NPES
