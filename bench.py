@@ -8,9 +8,11 @@ of its 128 query rows with the softmax state in registers and writes O and LSE a
 Prints one JSON line.  `value` is algorithmic TFLOP/s (4*B*H*d*visible (q,k) pairs per forward)
 over the wall time of K steps; `roofline` prices the block-attention launch of the same forward
 against the dense MFMA peak, timed by an event pair on the launch stream (a second pass of K
-forwards on a plan with the timing flag); `forward_with_step_partials` is the same forward on a
-plan that keeps the ring steps apart (a partial (O, LSE) per step, merged at the end of each
-workgroup; --step-partials makes that one the headline); `merge` times the merge kernel alone, on
+forwards on a plan with the timing flag); with --both-forwards, `forward_with_step_partials` is
+the same forward on a plan that keeps the ring steps apart (a partial (O, LSE) per step, merged
+at the end of each workgroup; --step-partials makes that one the headline, and every
+block-attention launch of a run without --both-forwards is of the headline kind, so a kernel
+trace of the run averages one kind of launch); `merge` times the merge kernel alone, on
 caller-held per-step partials, against HBM bandwidth; `cpu_baseline` is the CPU oracle timed on
 this host on a bounded sample of the same workload's rows.
 """
@@ -29,7 +31,12 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per block-kernel launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE): workload ->
 # (bytes, summary under profiles/, sha256[:16] of ringattn_kernels.hip when it was measured).  The figure is only
 # printed while the kernel source is still the one that was profiled.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    "cfg4": (4443e6, "profiles/block_attention_kernel_cfg4.md", "e57970fb4b43ea0b"),
+    "cfg2": (35.1e6, "profiles/block_attention_kernel_other_workloads.md", "e57970fb4b43ea0b"),
+    "cfg3": (8567e6, "profiles/block_attention_kernel_other_workloads.md", "e57970fb4b43ea0b"),
+    "cfg5": (40340e6, "profiles/block_attention_kernel_other_workloads.md", "e57970fb4b43ea0b"),
+}
 BASELINE_METRIC = "ring-attn fwd TFLOP/s + % bf16 MFMA peak, S=32K d=128 8-step ring, 1 GPU"
 
 
@@ -67,6 +74,7 @@ def main():
     ap.add_argument("--rank-local", action="store_true",
                     help="also time the ring rank by rank on rank-local buffers (one launch per rank and step)")
     ap.add_argument("--per-step", action="store_true", help="also time one block-attention launch per ring step")
+    ap.add_argument("--both-forwards", action="store_true", help="also time the forward of the other kind (see --step-partials)")
     ap.add_argument("--step-partials", action="store_true",
                     help="time the forward that keeps the ring steps apart (per-step partials in a workspace, merged at "
                          "the end) instead of the one that carries the softmax state through the steps")
@@ -142,19 +150,22 @@ def main():
     timed.close()
 
     # ---- the other forward (steps kept apart unless --step-partials, which swaps the two)
-    other = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=w.graph, layout=args.layout,
-                              half_partials=w.half_partials, step_partials=not args.step_partials)
-    for _ in range(2):
-        other.forward(qd, kd, vd, out, lse, stream)
-    ev0.record(stream)
-    for _ in range(args.steps):
-        other.forward(qd, kd, vd, out, lse, stream)
-    ev1.record(stream)
-    torch.cuda.synchronize()
-    other_ms = ev0.elapsed_time(ev1) / args.steps
-    other_leg = {"ms_per_step_events": round(other_ms, 4), "tflops": round(w.flops / (other_ms * 1e-3) / 1e12, 2),
-                 "workspace_bytes": int(other.lib.ringattn_workspace_bytes(other.params))}
-    other.close()
+    other_leg = None
+    if args.both_forwards:
+        other = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=w.graph, layout=args.layout,
+                                  half_partials=w.half_partials, step_partials=not args.step_partials)
+        for _ in range(2):
+            other.forward(qd, kd, vd, out, lse, stream)
+        ev0.record(stream)
+        for _ in range(args.steps):
+            other.forward(qd, kd, vd, out, lse, stream)
+        ev1.record(stream)
+        torch.cuda.synchronize()
+        other_ms = ev0.elapsed_time(ev1) / args.steps
+        other_leg = {"ms_per_step_events": round(other_ms, 4), "tflops": round(w.flops / (other_ms * 1e-3) / 1e12, 2),
+                     "workspace_bytes": int(other.lib.ringattn_workspace_bytes(other.params)),
+                     "partials": "none" if args.step_partials else ("fp16" if w.half_partials else "fp32")}
+        other.close()
 
     # ---- merge kernel alone: the ring merge on caller-held partials (random numbers: only the
     # bytes matter), events on the launch stream
