@@ -29,7 +29,10 @@
  * tests/test_oracle.py against independent routines (torch CPU fp64
  * matmul/softmax, scipy logsumexp), closed forms (Q = 0, constant V, causal
  * row 0, a dominant key), brute force on tiny shapes and algebraic invariants
- * (order independence of the ring, merge identity/commutativity).
+ * (order independence of the ring, merge identity/commutativity); the causal
+ * ring partials step by step, a block partial with a shifted diagonal and the
+ * rounded-probability form against scipy softmax / logsumexp on explicitly
+ * masked scores.
  *
  * Build: gcc -O3 -fopenmp -shared -fPIC (see oracle/build.py).
  */
