@@ -3,8 +3,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4]
 
 A step is one full forward of the workload: every ring step of every virtual rank, with Q/K/V
-already resident in HBM -- one block-attention launch in which a workgroup walks all ring steps
-of its 128 query rows with the softmax state in registers and writes O and LSE at the end.
+already resident in HBM -- one launch (ring_walk_kernel) in which a workgroup walks all ring steps
+of its 256 query rows with the softmax state in registers and writes O and LSE at the end.
 Prints one JSON line.  `value` is algorithmic TFLOP/s (4*B*H*d*visible (q,k) pairs per forward)
 over the wall time of K steps; `roofline` prices the block-attention launch of the same forward
 against the dense MFMA peak, timed by an event pair on the launch stream (a second pass of K
@@ -28,9 +28,9 @@ sys.path.insert(0, ROOT)
 # Published MI355X dense peaks used for the roofline (not the 2:1-sparsity figures)
 PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0}
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per block-kernel launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE): workload ->
-# (bytes, summary under profiles/, sha256[:16] of ringattn_kernels.hip when it was measured).  The figure is only
-# printed while the kernel source is still the one that was profiled.
+# HBM bytes per launch of the default forward's kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE): workload ->
+# (bytes, summary under profiles/, kernel_source_id() when it was measured).  The figure is only printed while the
+# kernel source is still the one that was profiled.
 MEASURED_TRAFFIC = {
     "cfg4": (4443e6, "profiles/block_attention_kernel_cfg4.md", "e57970fb4b43ea0b"),
     "cfg2": (35.1e6, "profiles/block_attention_kernel_other_workloads.md", "e57970fb4b43ea0b"),
@@ -41,13 +41,16 @@ BASELINE_METRIC = "ring-attn fwd TFLOP/s + % bf16 MFMA peak, S=32K d=128 8-step 
 
 
 def kernel_source_id():
+    """Hash of the sources of the kernel the default forward runs (ring_walk_kernel)."""
     import hashlib
-    path = os.path.join(ROOT, "ringattention_amd", "csrc", "ringattn_kernels.hip")
+    h = hashlib.sha256()
     try:
-        with open(path, "rb") as f:
-            return hashlib.sha256(f.read()).hexdigest()[:16]
+        for name in ("ringattn_walk.hip", "ringattn_device.h"):
+            with open(os.path.join(ROOT, "ringattention_amd", "csrc", name), "rb") as f:
+                h.update(f.read())
     except OSError:
         return None
+    return h.hexdigest()[:16]
 
 
 def describe(w):
@@ -140,7 +143,7 @@ def main():
         else:
             traffic_source = f"stale: {t_profile} was measured on kernel source {t_src}, this is {kernel_source_id()}"
     roofline = {
-        "kernel": "block_attention_kernel", "bound": "mfma",
+        "kernel": "block_attention_kernel" if args.step_partials else "ring_walk_kernel", "bound": "mfma",
         "achieved": round(block_tflops, 2), "peak": peak, "unit": "TFLOP/s", "frac": round(block_tflops / peak, 4),
         "traffic": traffic, "traffic_source": traffic_source,
         "launches_per_step": n_launch, "avg_launch_ms": round(avg_launch_ms, 4),

@@ -6,7 +6,8 @@
 
 namespace ringattn {
 
-constexpr int kBlockM = 128;  // query rows per workgroup (4 waves x 32 rows)
+constexpr int kBlockM = 128;  // query rows per workgroup of block_attention_kernel (4 waves x 32 rows)
+constexpr int kWalkM = 256;   // query rows per workgroup of ring_walk_kernel (8 waves x 32 rows)
 constexpr int kMaxParts = 64; // partial slots a merge can combine
 
 // One unit of block-attention work as the host layer lists it: the queries
@@ -77,7 +78,7 @@ struct BlockArgs {
   int64_t bh_stride;   // elements between heads of q and out (= S * D)
   int64_t kv_bh_stride;      // elements between heads of k and v
   int S;               // rows per head of q, out and lse
-  int q_tiles_max;     // kBlockM-row q tiles of the longest segment (grid dimension)
+  int q_tiles_max;     // q tiles (kBlockM rows; kWalkM for launch_walk) of the longest segment (grid dimension)
   int n_segs;
   int BH;              // batch * heads
   int heads;           // query heads per batch entry
@@ -120,6 +121,8 @@ struct TablePack {
 
 // dtype: 0 = fp16, 1 = bf16.  Return hipSuccess or the launch error.
 hipError_t launch_block(const BlockArgs& a, int dtype, int dim, hipStream_t stream);
+// the same work in kBlockCarryState mode by ring_walk_kernel (ringattn_walk.hip): 256-row q tiles, two-phase blocks
+hipError_t launch_walk(const BlockArgs& a, int dtype, int dim, hipStream_t stream);
 hipError_t launch_merge(const MergeArgs& a, int dtype, int dim, hipStream_t stream);
 // writes pack.seg to *seg_dst and pack.items[0..n) to item_dst
 hipError_t launch_write_table(const TablePack& pack, int n, Segment* seg_dst, SegItem* item_dst, hipStream_t stream);

@@ -1,0 +1,447 @@
+// gfx950 (CDNA4) kernel: the ring-attention forward with the softmax state carried through the
+// ring steps, in its two-phase form.
+//
+//   ring_walk_kernel : a workgroup of EIGHT waves owns 256 query rows of a segment (one head),
+//       keeps their Q in registers and walks the KV chunks those rows meet with the running max,
+//       sum and acc-O in registers from the first chunk to the last, as the reference's CTA does
+//       across its ring steps (csrc/ring_attention.cu:439-443,456,597); O = acc / l
+//       (:621-664) and LSE are written once.  The arithmetic per tile is that of
+//       block_attention_kernel (ringattn_kernels.hip): S^T = K Q^T and O^T += V^T P^T on
+//       v_mfma_f32_32x32x16, online softmax with a lazy reference max, K/V tiles through two
+//       4-deep LDS rings filled by direct-to-LDS loads, one barrier per two tiles.
+//
+//       What differs is how a tile's work is laid out in time.  The eight waves sit two per SIMD
+//       (wave w and wave w + 4).  Per tile every wave has an MFMA phase (O^T += V(u)^T P(u)^T, then
+//       S^T(u+1) = K(u+1) Q^T: 16 MFMAs and their 24 fragment reads from LDS at d = 128) and a
+//       softmax phase (row max, reference move, exponentials, row sum, conversion of P: VALU
+//       only).  Waves 0-3 run MFMA phase then softmax phase, waves 4-7 softmax phase then MFMA
+//       phase, between the same barriers: while one wave of a SIMD keeps the matrix pipe busy the
+//       other keeps the VALU busy, instead of both mixing the two kinds of work and colliding.
+//       Measured on synthetic tiles (same instruction mix, barrier and loads): 63.6 % of the
+//       MFMA-only rate against 53.4 % for the mixed stream.
+#include "ringattn_device.h"
+
+#include <type_traits>
+
+namespace ringattn {
+
+template <int DT, int D>
+__global__ __launch_bounds__(512, 1) void ring_walk_kernel(const BlockArgs a) {
+  using E = Elem<DT>;
+  constexpr int WAVES = 8;
+  constexpr int BM = kWalkM;       // query rows per workgroup: 8 waves x 32
+  constexpr int BN = 32;           // keys per tile
+  constexpr int NBUF = 4;          // ring depth of the K and of the V tiles
+  constexpr int CPR = D / 8;       // 16-byte chunks per row
+  constexpr int ROWB = D * 2;      // bytes per row
+  constexpr int TILE = BN * ROWB;  // bytes per tile
+  constexpr int KS = D / 16;       // contraction slices of QK^T
+  constexpr int DB = D / 32;       // 32-wide blocks of the head dim in PV
+  constexpr int PIECES = TILE / 1024;  // 1 KB wave-loads per tile: 8 at d = 128, 4 at d = 64
+  constexpr float kLazyLog2 = 8.f;
+  static_assert(BM == 32 * WAVES, "one 32-row block per wave");
+  static_assert(PIECES == WAVES || 2 * PIECES == WAVES, "a tile is loaded by all waves, or K and V by half of them each");
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * NBUF * TILE];  // K ring, V ring
+
+  const unsigned smem_base = lds_offset(smem);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+
+  Segment seg;
+  int bh, qt;
+  if (!decode_job<BM>(a, seg, bh, qt)) return;
+  const int q_start = seg.q_start, q_len = seg.q_len;
+  const int n_items = seg.item_count;
+  // items in run order: table order, except that item `last_item` is moved to the end
+  auto item_at = [&](int i) -> const SegItem* {
+    int idx = i;
+    if (seg.last_item >= 0) idx = (i == n_items - 1) ? seg.last_item : (i >= seg.last_item ? i + 1 : i);
+    return a.items + seg.item_begin + idx;
+  };
+
+  const int64_t head_off = (int64_t)bh * a.bh_stride;
+  // grouped-query attention: query head h of a batch entry reads KV head h / kv_group
+  const int kv_bh = (bh / a.heads) * (a.heads / a.kv_group) + (bh % a.heads) / a.kv_group;
+  const int64_t kv_head_off = (int64_t)kv_bh * a.kv_bh_stride;
+  const char* qbase = (const char*)a.q + (head_off + (int64_t)(q_start + qt * BM) * D) * 2;
+
+  // this lane's query row (local to the q tile): 32 wave + n; rows beyond the range read the last valid row
+  s16x8 qf[KS];
+  {
+    const int ql = min(qt * BM + 32 * wave + n, q_len - 1) - qt * BM;
+    const char* qrow = qbase + (int64_t)ql * ROWB + h * 16;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const s16x8*)(qrow + ks * 32);
+  }
+  // the 1 KB piece of a tile this wave loads: all waves a piece of K and of V each (d = 128), or waves 0-3 the
+  // K tile and waves 4-7 the V tile (d = 64)
+  const bool loads_k = PIECES == WAVES || wave < PIECES;
+  const bool loads_v = PIECES == WAVES || wave >= WAVES - PIECES;
+  const int piece_k = wave, piece_v = PIECES == WAVES ? wave : wave - (WAVES - PIECES);
+  int goff_k, goff_v;
+  {
+    const int pk = piece_k * 64 + lane, pv = piece_v * 64 + lane;
+    goff_k = (pk / CPR) * ROWB + (((pk % CPR) ^ k_swizzle<D>(pk / CPR)) << 4);
+    goff_v = (pv / CPR) * ROWB + (((pv % CPR) ^ v_swizzle<D>(pv / CPR)) << 4);
+  }
+  int koff[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) koff[ks] = n * ROWB + (((2 * ks + h) ^ k_swizzle<D>(n)) << 4);
+  int voff[DB];
+  {
+    const int s = lane & 15, g1 = (lane >> 4) & 1;
+    const int row8 = 4 * h + (s >> 2);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int c = 2 * (2 * db + g1) + ((s & 3) >> 1);
+      voff[db] = row8 * ROWB + ((c ^ v_swizzle<D>(row8)) << 4) + ((s & 1) << 3);
+    }
+  }
+
+  float m = -INFINITY;  // reference max (raw score units)
+  float ms = 0.f;       // m * k2, 0 while m is -inf (guard of csrc/ring_attention.cu:183)
+  float ls[4] = {0.f, 0.f, 0.f, 0.f};
+  f32x16 oacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
+  f32x16 sacc;   // scores of the tile in flight: written by an MFMA phase, consumed by the next softmax phase
+  s16x8 pf[2];   // its probabilities in B-operand layout: written by a softmax phase, consumed by the next MFMA phase
+
+  // ---- the KV chunk being walked (wave-uniform)
+  const char *kbase = nullptr, *vbase = nullptr;
+  // where the loads that run past the last tile go: the first tiles of the next chunk when
+  // the pipeline carries over (stride TILE), else a re-read of the last tile (stride 0)
+  int64_t past_delta = 0;  // from the end of this chunk's K (V) to that place
+  int past_stride = 0;
+  int kv_len = 0, n_tiles = 0, first_masked = 0, kv_tail = -1, diag_rows = 0;
+  bool diag = false;
+  auto set_chunk = [&](const SegItem* w) {
+    diag = w->diag_off >= 0;
+    kv_len = w->kv_len;
+    diag_rows = w->diag_off + qt * BM;  // keys below this local index are visible to the whole q tile
+    const int kv_tiles = (kv_len + BN - 1) / BN;
+    kv_tail = (kv_len % BN) ? kv_len / BN : -1;  // the tile with surplus keys, if any
+    n_tiles = diag ? min(kv_tiles, (diag_rows + BM + BN - 1) / BN) : kv_tiles;
+    // tiles >= first_masked need a mask (causal diagonal or surplus keys)
+    first_masked = min(diag ? diag_rows / BN : n_tiles, kv_tail >= 0 ? kv_tail : n_tiles);
+    kbase = (const char*)a.k + (kv_head_off + (int64_t)w->kv_start * D) * 2;
+    vbase = (const char*)a.v + (kv_head_off + (int64_t)w->kv_start * D) * 2;
+  };
+  // bytes to step back so that a row of tile kv_tail beyond the KV range reads the last valid row
+  auto surplus = [&](int piece) {
+    const int row = (piece * 64 + lane) / CPR;
+    return max(0, kv_tail * BN + row - (kv_len - 1)) * ROWB;
+  };
+  // byte offset of tile t from the chunk's first tile, branch-free: t < n_tiles gives t TILE; beyond that
+  // n_tiles TILE + past_delta + (t - n_tiles) past_stride
+  auto tile_offset = [&](int t) -> int64_t {
+    const int64_t beyond = (int64_t)((n_tiles - 1 - t) >> 31);  // all ones iff t >= n_tiles
+    return (int64_t)min(t, n_tiles) * TILE + (int64_t)max(t - n_tiles, 0) * past_stride + (past_delta & beyond);
+  };
+  // `checked`: the tile may be kv_tail (steady blocks never issue that one)
+  auto issue_k = [&](int t, auto checked) {
+    if (!loads_k) return;
+    const char* kt = kbase + tile_offset(t);
+    const unsigned kd = __builtin_amdgcn_readfirstlane(smem_base + (t & (NBUF - 1)) * TILE + piece_k * 1024);
+    if (decltype(checked)::value && t == kv_tail) load_lds_16(kt, goff_k - surplus(piece_k), kd);
+    else load_lds_16(kt, goff_k, kd);
+  };
+  auto issue_v = [&](int t, auto checked) {
+    if (!loads_v) return;
+    const char* vt = vbase + tile_offset(t);
+    const unsigned vd = __builtin_amdgcn_readfirstlane(smem_base + (NBUF + (t & (NBUF - 1))) * TILE + piece_v * 1024);
+    if (decltype(checked)::value && t == kv_tail) load_lds_16(vt, goff_v - surplus(piece_v), vd);
+    else load_lds_16(vt, goff_v, vd);
+  };
+  constexpr std::true_type kChecked{};
+  constexpr std::false_type kUnchecked{};
+
+  // S^T = K Q^T of one 32-key tile (csrc/ring_attention.cu:565)
+  auto qk = [&](int kslot) {
+    const unsigned char* ks_lds = smem + kslot * TILE;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) sacc[e] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const s16x8 kfr = *(const s16x8*)(ks_lds + koff[ks]);
+      sacc = E::mma(kfr, qf[ks], sacc);
+    }
+  };
+  // key visible iff inside the KV range and key_local <= query_local + diag_off
+  auto mask_tile = [&](int t, auto always) {
+    if (decltype(always)::value || t >= first_masked) {
+      int lim = kv_len - 1 - t * BN - 4 * h;
+      if (diag) lim = min(lim, diag_rows + 32 * wave + n - t * BN - 4 * h);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int key = 8 * (e >> 2) + (e & 3);
+        if (key > lim) sacc[e] = -INFINITY;
+      }
+    }
+  };
+  // max(m, row max of the tile): two chains of max(max(x, a), b), each link one v_max3_f32; one
+  // exchange between the halves of the wave
+  auto tile_max = [&]() {
+    float m0 = m, m1 = m;
+#pragma unroll
+    for (int e = 0; e < 16; e += 4) {
+      m0 = fmaxf(fmaxf(m0, sacc[e]), sacc[e + 1]);
+      m1 = fmaxf(fmaxf(m1, sacc[e + 2]), sacc[e + 3]);
+    }
+    return cross_half_max(fmaxf(m0, m1));
+  };
+  // The reference max moves when some row's cand = max(m, tile max) is far above it (or it is still
+  // unset): rescale of l and acc-O as in csrc/ring_attention.cu:226-232.
+  auto move_reference = [&](float cand) {
+    const bool far = (cand - m) * a.scale_log2 > kLazyLog2;
+    if (__builtin_amdgcn_ballot_w64(far) != 0) {
+      const float cs = (cand == -INFINITY) ? 0.f : cand * a.scale_log2;
+      const float alpha = __builtin_amdgcn_exp2f(m * a.scale_log2 - cs);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ls[i] *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) oacc[db] *= alpha;
+      m = cand;
+      ms = cs;
+    }
+  };
+  // P^T = exp2(S^T k2 - m k2): row sum from the unrounded values (csrc/ring_attention.cu:242),
+  // MFMA operands rounded to the storage type (:604)
+  auto exponentials = [&]() {
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      typename E::vec8 pv;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * t2 + e], a.scale_log2, -ms));
+        ls[e & 3] += p;
+        pv[e] = (typename E::type)p;
+      }
+      pf[t2] = __builtin_bit_cast(s16x8, pv);
+    }
+  };
+  // O^T += V^T P^T of one 32-key tile (csrc/ring_attention.cu:609)
+  auto pv_product = [&](int vslot) {
+    const unsigned char* vs_lds = smem + (NBUF + vslot) * TILE;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      const unsigned char* vrow = vs_lds + 16 * t2 * ROWB;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vrow + voff[db]));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vrow + 8 * ROWB + voff[db]));
+        const s16x8 vfr = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        oacc[db] = E::mma(vfr, pf[t2], oacc[db]);
+      }
+    }
+  };
+  // the softmax phase of the tile whose scores are in sacc
+  auto softmax_phase = [&]() {
+    move_reference(tile_max());
+    exponentials();
+  };
+  auto phase_fence = [&]() { __builtin_amdgcn_sched_barrier(0); };  // keeps the compiler from mixing the phases
+  // The MFMA phase of a steady block: O += P(u) V(u), then S(u+1) = K(u+1) Q^T.  Scheduling hint: the
+  // fragment reads run ahead of the MFMAs that consume them (8 reads up front, two more behind each of
+  // the PV MFMAs: the K fragments are all on their way when the QK MFMAs start), so the matrix pipe does
+  // not wait for LDS latency inside the phase.
+  auto mfma_phase = [&](int vslot, int kslot) {
+    pv_product(vslot);
+    qk(kslot);
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+    for (int i = 0; i < 2 * DB; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < KS; ++i) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+  };
+  auto ring_barrier = [&]() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  };
+
+  // The walk of all items, for one half of the workgroup.  At the start of block u the waves of the
+  // first half hold P(u) (their softmax phase of tile u is done), those of the second half the raw
+  // scores S(u).  Block u: the even ones start with the barrier of the pair (u, u+1) -- K(u+1),
+  // K(u+2), V(u), V(u+1), issued during the previous pair, have landed, and every wave is past
+  // block u-1, so the ring slots of K(u-1), K(u), V(u-2), V(u-1) are free for K(u+3), K(u+4),
+  // V(u+2), V(u+3), which are issued during this pair -- then
+  //     first half :  O += P(u) V(u), S(u+1) = K(u+1) Q^T  |  softmax of S(u+1)
+  //     second half:  softmax of S(u)                      |  O += P(u) V(u), S(u+1) = K(u+1) Q^T
+  auto walk = [&](auto second_c) {
+    constexpr bool SECOND = decltype(second_c)::value;
+    // STEADY blocks (tiles u+1 and u+2 unmasked or covered by MASKED) have compile-time ring slots
+    auto block = [&](auto slot_c, auto steady, auto masked, int u) {
+      constexpr int SLOT = decltype(slot_c)::value;  // u mod 4 (STEADY only)
+      constexpr bool STEADY = decltype(steady)::value;
+      constexpr bool MASKED = decltype(masked)::value;  // STEADY only: tile u+1 gets the mask
+      if (STEADY) {
+        // the two tile loads of a block go out next to the softmax phase of the wave (the VALU side has issue
+        // slots to spare): K(u+3), K(u+4) in even blocks, V(u+1), V(u+2) in odd ones
+        auto issue_loads = [&]() {
+          if ((SLOT & 1) == 0) {
+            issue_k(u + 3, kUnchecked);
+            issue_k(u + 4, kUnchecked);
+          } else {
+            issue_v(u + 1, kUnchecked);
+            issue_v(u + 2, kUnchecked);
+          }
+        };
+        if ((SLOT & 1) == 0) ring_barrier();
+        if (SECOND) issue_loads();
+        phase_fence();
+        if (!SECOND) {
+          mfma_phase(SLOT, (SLOT + 1) & 3);
+          if (MASKED) mask_tile(u + 1, kChecked);
+        } else {
+          softmax_phase();
+        }
+        phase_fence();
+        if (!SECOND) issue_loads();
+        phase_fence();
+        if (!SECOND) {
+          // the scores past the end of a chunk belong to the next chunk (or to nothing): its start handles them
+          if (u + 1 < n_tiles) softmax_phase();
+        } else {
+          mfma_phase(SLOT, (SLOT + 1) & 3);
+          if (MASKED) mask_tile(u + 1, kChecked);
+        }
+        phase_fence();
+      } else {
+        if ((u & 1) == 0) {
+          ring_barrier();
+          if (u + 3 < n_tiles) issue_k(u + 3, kChecked);
+          if (u + 4 < n_tiles) issue_k(u + 4, kChecked);
+          if (u + 2 < n_tiles) issue_v(u + 2, kChecked);
+          if (u + 3 < n_tiles) issue_v(u + 3, kChecked);
+        }
+        if (SECOND) softmax_phase();
+        pv_product(u & 3);
+        if (u + 1 < n_tiles) {
+          qk((u + 1) & 3);
+          mask_tile(u + 1, kUnchecked);
+          if (!SECOND) softmax_phase();
+        }
+      }
+    };
+
+    using C0 = std::integral_constant<int, 0>;
+    using C1 = std::integral_constant<int, 1>;
+    using C2 = std::integral_constant<int, 2>;
+    using C3 = std::integral_constant<int, 3>;
+
+    bool carried = false;  // the previous chunk's pipeline ran on into this one
+    for (int it = 0; it < n_items; ++it) {
+      const SegItem* w = item_at(it);
+      set_chunk(w);
+      // The pipeline carries over into the next chunk when this one ends in plain steady groups
+      // on a multiple of four tiles (ring slots then line up with a fresh start) and the next
+      // chunk has its first three tiles in full.
+      bool carry = false;
+      if (it + 1 < n_items) {
+        const SegItem* wn = item_at(it + 1);
+        carry = !diag && kv_tail < 0 && (n_tiles & 3) == 0 && wn->kv_len >= 4 * BN;
+        if (carry) {
+          past_delta = ((int64_t)wn->kv_start - w->kv_start) * ROWB - (int64_t)n_tiles * TILE;
+          past_stride = TILE;
+        }
+      }
+      if (!carry) {
+        past_delta = -(int64_t)TILE;
+        past_stride = 0;
+      }
+
+      if (!carried) {
+        if (it > 0) __syncthreads();  // every wave is done with the ring slots of the previous chunk
+        // the first tiles go out next to the Q loads: one memory latency for all of them
+        issue_k(0, kChecked);
+        if (n_tiles > 1) issue_k(1, kChecked);
+        if (n_tiles > 2) issue_k(2, kChecked);
+        issue_v(0, kChecked);
+        if (n_tiles > 1) issue_v(1, kChecked);
+        __builtin_amdgcn_s_waitcnt(0);  // retire the Q loads with a wait the compiler can see (and the tiles)
+        ring_barrier();
+        qk(0);
+      }
+      // (carried: the last block of the previous chunk left the scores of tile 0 in sacc; K(1), K(2),
+      // V(0), V(1) are in flight)
+      mask_tile(0, kUnchecked);
+      if (!SECOND) softmax_phase();
+
+      // Steady blocks come in groups of four.  A group starting at u computes the scores of tiles
+      // u+1 .. u+4 and loads up to tile u+6:
+      //   plain groups   while those four tiles need no mask; without any mask in the chunk the last
+      //                  group runs up to tile n_tiles-1 and its last block computes the scores of
+      //                  the tile after the last one (the next chunk's first, or nothing of use);
+      //   masked groups  (diagonal chunks) for the rest: every block masks its tile u+1;
+      //   a chunk with surplus keys in its last tile keeps clear of that tile (its loads need the
+      //   clamped form) and leaves the rest to the general blocks.
+      const bool ragged = kv_tail >= 0;
+      const int plain_end = ragged ? min(first_masked, kv_tail - 2) : (diag ? first_masked : n_tiles + 1);
+      const int masked_end = (diag && !ragged) ? n_tiles + 1 : 0;
+      int u = 0;
+      for (; u + 4 < plain_end; u += 4) {
+        block(C0{}, std::true_type{}, std::false_type{}, u);
+        block(C1{}, std::true_type{}, std::false_type{}, u + 1);
+        block(C2{}, std::true_type{}, std::false_type{}, u + 2);
+        block(C3{}, std::true_type{}, std::false_type{}, u + 3);
+      }
+      for (; u + 4 < masked_end; u += 4) {
+        block(C0{}, std::true_type{}, std::true_type{}, u);
+        block(C1{}, std::true_type{}, std::true_type{}, u + 1);
+        block(C2{}, std::true_type{}, std::true_type{}, u + 2);
+        block(C3{}, std::true_type{}, std::true_type{}, u + 3);
+      }
+      for (; u < n_tiles; ++u) block(C0{}, std::false_type{}, std::false_type{}, u);
+      if (!carry) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // re-reads of the last tile
+      carried = carry;
+    }
+  };
+  if (wave < WAVES / 2) walk(std::false_type{});
+  else walk(std::true_type{});
+
+  // the rows' result: the reference's epilogue (csrc/ring_attention.cu:621-664), O = acc / l in the
+  // storage type, plus the LSE
+  {
+    const float l = cross_half_sum((ls[0] + ls[1]) + (ls[2] + ls[3]));
+    const float inv = (l > 0.f) ? 1.f / l : 0.f;
+    const int row_l = qt * BM + 32 * wave + n;
+    if (row_l < q_len) {  // not a row beyond the query range
+      const int64_t row = (int64_t)bh * a.S + q_start + row_l;
+      typename E::type* orow = (typename E::type*)a.out + row * D;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          typename E::vec4 val;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) val[e] = (typename E::type)(oacc[db][4 * q4 + e] * inv);
+          *(typename E::vec4*)(orow + 32 * db + 8 * q4 + 4 * h) = val;
+        }
+      if (h == 0 && a.lse) a.lse[row] = (l > 0.f) ? (ms + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
+    }
+  }
+}
+
+hipError_t launch_walk(const BlockArgs& a, int dtype, int dim, hipStream_t stream) {
+  if (a.n_segs <= 0) return hipSuccess;
+  if (a.mode != kBlockCarryState) return hipErrorInvalidValue;
+  const int q_tiles = a.q_tiles_max;  // kWalkM-row tiles of the longest segment
+  const int64_t groups = (int64_t)a.n_segs * a.BH;
+  const int64_t blocks = (a.groups ? (int64_t)a.groups_per_xcd : (groups + 7) / 8) * 8 * q_tiles;
+  if (q_tiles <= 0 || blocks > INT32_MAX) return hipErrorInvalidValue;
+  const unsigned grid = (unsigned)blocks;
+  if (dtype == 0 && dim == 64) ring_walk_kernel<0, 64><<<grid, 512, 0, stream>>>(a);
+  else if (dtype == 0 && dim == 128) ring_walk_kernel<0, 128><<<grid, 512, 0, stream>>>(a);
+  else if (dtype == 1 && dim == 64) ring_walk_kernel<1, 64><<<grid, 512, 0, stream>>>(a);
+  else if (dtype == 1 && dim == 128) ring_walk_kernel<1, 128><<<grid, 512, 0, stream>>>(a);
+  else return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+}  // namespace ringattn

@@ -1,7 +1,8 @@
-"""What the compiler made of the block kernel: the d = 128 instantiations must keep two waves
-per SIMD (256 registers) and their steady key loops -- the loops that hold 64 MFMAs, four
-32-key blocks -- must not touch scratch memory.  (The kernel as a whole does spill a few values
-around the chunk prologue and the general, non-unrolled blocks; those run once per chunk.)
+"""What the compiler made of the attention kernels: the d = 128 instantiations must keep two
+waves per SIMD (256 registers) and their steady key loops -- the loops that hold 64 MFMAs, four
+32-key blocks -- must not touch scratch memory.  (block_attention_kernel as a whole does spill a
+few values around the chunk prologue and the general, non-unrolled blocks; those run once per
+chunk.  ring_walk_kernel must not spill at all.)
 Compiles the kernels to assembly for gfx950; needs hipcc but no GPU."""
 import os
 import re
@@ -42,19 +43,18 @@ def loops_of(asm):
     return out
 
 
-def test_steady_key_loops_are_spill_free_at_two_waves_per_simd(tmp_path):
+def compile_to_asm(source, out):
+    """Assembly of one kernel source plus the compiler's per-kernel resource remarks."""
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
         pytest.skip("no hipcc")
     from ringattention_amd import _build
-    src = os.path.join(_build.CSRC, "ringattn_kernels.hip")
-    out = tmp_path / "kernels.s"
+    src = os.path.join(_build.CSRC, source)
     flags = [f for f in _build.HIPCC_FLAGS if f not in ("-shared", "-fPIC", "-pthread")]
     res = subprocess.run([hipcc] + flags + ["-S", "--cuda-device-only", "-Rpass-analysis=kernel-resource-usage",
                                             "-I", os.path.join(ROOT, "include"), "-I", _build.CSRC, src, "-o", str(out)],
                          capture_output=True, text=True, timeout=900)
     assert res.returncode == 0, res.stderr[-2000:]
-    # occupancy and register count from the compiler's remarks
     usage = {}
     name = None
     for line in res.stderr.split("\n"):
@@ -66,6 +66,32 @@ def test_steady_key_loops_are_spill_free_at_two_waves_per_simd(tmp_path):
             m = re.search(re.escape(key) + r": (\d+)", line)
             if m and name:
                 usage[name][key] = int(m.group(1))
+    return out.read_text(), usage
+
+
+def steady_loops(asm, kernel):
+    start = asm.index("\n" + kernel + ":")
+    end = asm.index(".amdhsa_kernel " + kernel, start)
+    return [(lab, ins) for lab, ins in loops_of(asm[start:end]) if sum(i.startswith("v_mfma") for i in ins) == 64]
+
+
+def test_walk_kernel_runs_two_waves_per_simd_without_spills(tmp_path):
+    asm, usage = compile_to_asm("ringattn_walk.hip", tmp_path / "walk.s")
+    walks = {n: u for n, u in usage.items() if "ring_walk_kernel" in n}
+    assert len(walks) == 4                                     # {fp16, bf16} x {64, 128}
+    for n, u in walks.items():
+        assert u["ScratchSize [bytes/lane]"] == 0, (n, u)
+        assert u["VGPRs"] <= 256, (n, u)                       # eight waves per workgroup, one workgroup per compute unit
+        assert u["LDS Size [bytes/block]"] == (65536 if "Li128E" in n else 32768), (n, u)
+        if "Li128E" in n:
+            steady = steady_loops(asm, n)
+            assert len(steady) == 4, (n, len(steady))          # plain and masked groups, for each half of the workgroup
+            for lab, ins in steady:
+                assert sum(i.startswith("s_barrier") for i in ins) == 2, (n, lab)   # one barrier per two tiles
+
+
+def test_steady_key_loops_are_spill_free_at_two_waves_per_simd(tmp_path):
+    asm, usage = compile_to_asm("ringattn_kernels.hip", tmp_path / "kernels.s")
     blocks = {n: u for n, u in usage.items() if "block_attention_kernel" in n}
     assert len(blocks) == 8                                    # {fp16, bf16} x {64, 128} x {fp32, fp16 partials}
     for n, u in blocks.items():
@@ -73,14 +99,11 @@ def test_steady_key_loops_are_spill_free_at_two_waves_per_simd(tmp_path):
         assert u["VGPRs"] <= 256, (n, u)
         if "Li128E" in n:
             assert u["LDS Size [bytes/block]"] == 65536, (n, u)   # two workgroups per compute unit
-    asm = out.read_text()
     checked = 0
     for n in blocks:
         if "Li128E" not in n:
             continue
-        start = asm.index("\n" + n + ":")
-        end = asm.index(".amdhsa_kernel " + n, start)
-        steady = [(lab, ins) for lab, ins in loops_of(asm[start:end]) if sum(i.startswith("v_mfma") for i in ins) == 64]
+        steady = steady_loops(asm, n)
         assert len(steady) == 2, (n, len(steady))              # the plain and the masked groups of four blocks
         for lab, ins in steady:
             assert not any(i.startswith("scratch_") for i in ins), (n, lab)
