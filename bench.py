@@ -32,10 +32,10 @@ PEAK_HBM_GBS = 8000.0
 # (bytes, summary under profiles/, kernel_source_id() when it was measured).  The figure is only printed while the
 # kernel source is still the one that was profiled.
 MEASURED_TRAFFIC = {
-    "cfg4": (4443e6, "profiles/block_attention_kernel_cfg4.md", "e57970fb4b43ea0b"),
-    "cfg2": (35.1e6, "profiles/block_attention_kernel_other_workloads.md", "e57970fb4b43ea0b"),
-    "cfg3": (8567e6, "profiles/block_attention_kernel_other_workloads.md", "e57970fb4b43ea0b"),
-    "cfg5": (40340e6, "profiles/block_attention_kernel_other_workloads.md", "e57970fb4b43ea0b"),
+    "cfg4": (3404e6, "profiles/ring_walk_kernel_cfg4.md", "b72efe25495fa5c4"),
+    "cfg2": (34.1e6, "profiles/ring_walk_kernel_other_workloads.md", "b72efe25495fa5c4"),
+    "cfg3": (2217e6, "profiles/ring_walk_kernel_other_workloads.md", "b72efe25495fa5c4"),
+    "cfg5": (18260e6, "profiles/ring_walk_kernel_other_workloads.md", "b72efe25495fa5c4"),
 }
 BASELINE_METRIC = "ring-attn fwd TFLOP/s + % bf16 MFMA peak, S=32K d=128 8-step ring, 1 GPU"
 
@@ -81,6 +81,9 @@ def main():
     ap.add_argument("--step-partials", action="store_true",
                     help="time the forward that keeps the ring steps apart (per-step partials in a workspace, merged at "
                          "the end) instead of the one that carries the softmax state through the steps")
+    ap.add_argument("--operands", default="workload", choices=["workload", "zeros"],
+                    help="diagnostic: 'zeros' runs the same launches on all-zero Q, K, V (same instruction stream, no operand "
+                         "toggling: shows what the power manager leaves of the clock); not a valid headline")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the cpu_baseline sample (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -97,6 +100,9 @@ def main():
 
     q, k, v = api.make_qkv_bits(w)
     qd, kd, vd = (api.bits_to_tensor(x, w.dtype) for x in (q, k, v))
+    if args.operands == "zeros":
+        for t in (qd, kd, vd):
+            t.zero_()
     plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=w.graph, layout=args.layout,
                              half_partials=w.half_partials, step_partials=args.step_partials)
     out = torch.empty_like(qd)
@@ -277,11 +283,12 @@ def main():
                          f"full forward extrapolates to {w.flops / (fl / dt):.0f} s"}
 
     print(json.dumps({
-        "metric": BASELINE_METRIC if (w.name == "cfg4" and args.layout == "contiguous")
-        else f"ring-attn fwd TFLOP/s + % {w.dtype} MFMA peak, {describe(w)}, {args.layout} layout, 1 GPU",
+        "metric": BASELINE_METRIC if (w.name == "cfg4" and args.layout == "contiguous" and args.operands == "workload")
+        else f"ring-attn fwd TFLOP/s + % {w.dtype} MFMA peak, {describe(w)}, {args.layout} layout, 1 GPU"
+        + ("" if args.operands == "workload" else ", ALL-ZERO OPERANDS (diagnostic)"),
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "ms_per_step_events": round(ms_per_step_events, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": w.dtype, "data": "synthetic",
+        "dtype": w.dtype, "data": "synthetic" if args.operands == "workload" else "all-zero operands (diagnostic, not the workload)",
         "config": {"workload": describe(w), "algorithmic_flop": w.flops, "graph": bool(w.graph), "layout": args.layout,
                    "partials": ("fp16" if w.half_partials else "fp32") if args.step_partials
                    else "none: softmax state carried through the ring steps in registers",
