@@ -53,13 +53,12 @@ struct Segment {
 };
 static_assert(sizeof(Segment) == 32, "Segment is read as two 16-byte scalar loads");
 
-// What a workgroup of the block kernel does with the softmax state (max, sum, acc-O) of its rows
-// between the KV chunks it walks.
+// What a workgroup does with the softmax state (max, sum, acc-O) of its rows between the KV chunks it walks.
 enum BlockMode {
-  kBlockPartials = 0,        // per chunk: emit the normalised partial (O, LSE), reset the state
-  kBlockPartialsMerged = 1,  // the same, and after the last chunk merge the partials of the rows into out / lse
+  kBlockPartials = 0,        // per chunk: emit the normalised partial (O, LSE), reset the state   (launch_block)
+  kBlockPartialsMerged = 1,  // the same, and after the last chunk merge the partials of the rows into out / lse   (launch_block)
   kBlockCarryState = 2,      // carry the state across the chunks, as the reference's CTA does across its ring
-                             // steps (csrc/ring_attention.cu:439-443,597), and write out / lse once: no partials
+                             // steps (csrc/ring_attention.cu:439-443,597), and write out / lse once: no partials   (launch_walk)
 };
 
 struct BlockArgs {

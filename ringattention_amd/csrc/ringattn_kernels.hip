@@ -1,11 +1,14 @@
-// gfx950 (CDNA4) kernels for the ring-attention forward path.
+// gfx950 (CDNA4) kernels for the ring-attention forward path: the ring steps kept apart.
+// (The forward that carries the softmax state through the steps is ring_walk_kernel,
+// ringattn_walk.hip.)
 //
 //   block_attention_kernel : the ring steps of every virtual rank.  A workgroup owns 128
 //       query rows, keeps their Q in registers and walks the KV chunks those rows meet (the
 //       reference's CTA loops over the ring steps in the same way, csrc/ring_attention.cu:
 //       439-443,456), per chunk
 //       S^T = K Q^T, online softmax with running max / sum, O^T += V^T P^T,
-//       emitting a normalised fp32 partial O and a natural-log fp32 LSE per chunk.
+//       emitting a normalised fp32 partial O and a natural-log fp32 LSE per chunk, and, when
+//       asked, merging the partials of its rows at the end.
 //       It restates the inner KV-tile loop of the reference kernel
 //       (csrc/ring_attention.cu:536-610: gemm_smem :278-301, softmax_rescale_o
 //       :194-245 completed with the missing `sum += sum_cur` tail,
@@ -680,37 +683,11 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockArgs
     }
   };
 
-  // the rows' final result from a state carried over every chunk: the reference's epilogue
-  // (csrc/ring_attention.cu:621-664), O = acc / l in the storage type, plus the LSE
-  auto emit_result = [&]() {
-#pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-      const float l = cross_half_sum((ls[qb][0] + ls[qb][1]) + (ls[qb][2] + ls[qb][3]));
-      const float inv = (l > 0.f) ? 1.f / l : 0.f;
-      const int row_l = qt * BM + 32 * QB * wave + 32 * qb + n;
-      if (row_l >= q_len) continue;  // a row beyond the query range
-      const int64_t row = (int64_t)bh * a.S + q_start + row_l;
-      typename E::type* orow = (typename E::type*)a.out + row * D;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          typename E::vec4 val;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) val[e] = (typename E::type)(oacc[qb][db][4 * q4 + e] * inv);
-          *(typename E::vec4*)(orow + 32 * db + 8 * q4 + 4 * h) = val;
-        }
-      if (h == 0 && a.lse) a.lse[row] = (l > 0.f) ? (ms[qb] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
-    }
-  };
-
   using C0 = std::integral_constant<int, 0>;
   using C1 = std::integral_constant<int, 1>;
   using C2 = std::integral_constant<int, 2>;
   using C3 = std::integral_constant<int, 3>;
 
-  const bool keep_state = a.mode == kBlockCarryState;
-  bool fresh = true;     // the softmax state is empty: the chunk's first tile sets the reference max
   bool carried = false;  // the previous chunk's pipeline ran on into this one
   for (int it = 0; it < n_items; ++it) {
     const SegItem* w = item_at(it);
@@ -752,8 +729,7 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockArgs
       float cand[QB];
       mask_tile(s_even, 0, kUnchecked);
       tile_maxes(s_even, cand);
-      if (fresh) set_reference(cand);
-      else move_reference(cand, true);
+      set_reference(cand);
     }
 
     // Steady blocks come in groups of four (ring slots are compile-time constants).  A group
@@ -785,13 +761,6 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockArgs
       else block(C0{}, std::false_type{}, std::false_type{}, u);
     }
     carried = carry;
-    if (keep_state) {
-      // the softmax state runs on into the next chunk; with the pipeline carried over as well,
-      // the chunk boundary is just another tile boundary
-      fresh = false;
-      if (!carry) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // re-reads of the last tile
-      continue;
-    }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next chunk's first tiles, or re-reads of the last tile
     if (carry) {
       __syncthreads();
@@ -800,11 +769,6 @@ __global__ __launch_bounds__(256, 2) void block_attention_kernel(const BlockArgs
     emit_partial(w);
     reset_state();
   }
-  if (keep_state) {
-    emit_result();
-    return;
-  }
-
   // ---- fused merge: this workgroup's rows over the partials it has just written
   if (a.mode == kBlockPartialsMerged) {
     static_assert(sizeof(smem) >= kMaxParts * BM * sizeof(float), "partial LSEs of a q tile fit the rings");
@@ -836,6 +800,7 @@ __global__ __launch_bounds__(64) void write_table_kernel(const TablePack pack, i
 // ---- host launchers -----------------------------------------------------------------
 hipError_t launch_block(const BlockArgs& a, int dtype, int dim, hipStream_t stream) {
   if (a.n_segs <= 0) return hipSuccess;
+  if (a.mode != kBlockPartials && a.mode != kBlockPartialsMerged) return hipErrorInvalidValue;  // carry mode: launch_walk
   const int q_tiles = a.q_tiles_max;
   const int64_t groups = (int64_t)a.n_segs * a.BH;
   const int64_t blocks = (a.groups ? (int64_t)a.groups_per_xcd : (groups + 7) / 8) * 8 * q_tiles;
