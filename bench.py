@@ -149,7 +149,7 @@ def main():
         else:
             traffic_source = f"stale: {t_profile} was measured on kernel source {t_src}, this is {kernel_source_id()}"
     roofline = {
-        "kernel": "block_attention_kernel" if args.step_partials else "ring_walk_kernel", "bound": "mfma",
+        "kernel": "ring_walk_kernel", "bound": "mfma",
         "achieved": round(block_tflops, 2), "peak": peak, "unit": "TFLOP/s", "frac": round(block_tflops / peak, 4),
         "traffic": traffic, "traffic_source": traffic_source,
         "launches_per_step": n_launch, "avg_launch_ms": round(avg_launch_ms, 4),

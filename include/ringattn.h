@@ -43,7 +43,7 @@ extern "C" {
 #define RINGATTN_DTYPE_BF16 1
 
 #define RINGATTN_MAX_NPES 64
-#define RINGATTN_TILE 128          /* query rows per workgroup: per-rank lengths may be any positive number and may differ between
+#define RINGATTN_TILE 256          /* query rows per workgroup: per-rank lengths may be any positive number and may differ between
                                       ranks (the tail predication the reference leaves open, csrc/ring_attention.cu:143-145);
                                       multiples of this waste no part of a tile */
 
@@ -125,7 +125,7 @@ int ringattn_plan_destroy(ringattn_plan* plan);
 /*
  * The whole forward for all npes virtual ranks: replaces ring_attention()
  * (csrc/ring_attention.cu:706-722) run on every PE.  ONE block-attention launch: a workgroup
- * owns 128 query rows and walks every ring step of those rows with the running max, sum and
+ * owns 256 query rows and walks every ring step of those rows with the running max, sum and
  * acc-O in registers, like the reference's CTA (:439-443,456,597), then writes O = acc / sum
  * (:621-664) and the LSE.  (With RINGATTN_FLAG_STEP_PARTIALS: a partial (O, LSE) per step into
  * the workspace, merged at the end of the workgroup.)

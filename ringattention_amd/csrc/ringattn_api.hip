@@ -139,7 +139,7 @@ struct HostSegment {
   int start = 0, len = 0;
   std::vector<ringattn::WorkItem> items;  // restricted to the segment: q_start = start, q_len = len
   uint64_t active = 0;                    // the steps (partial slots) of the items
-  int64_t tile_work = 0;                  // keys the busiest 128-row tile of the segment visits
+  int64_t tile_work = 0;                  // keys the busiest q tile of the segment visits
 };
 
 void rank_segments(std::vector<HostSegment>& out, const Derived& d, int P, bool causal, int r) {
@@ -204,8 +204,7 @@ size_t workspace_bytes_of(const ringattn_params* p, const Derived& d) {
 // A slice of the device tables: what one block launch runs.
 struct TableSlice {
   int seg_begin = 0, seg_count = 0;
-  int q_tiles_max = 0;  // kBlockM-row tiles of the longest segment
-  int max_q_len = 0;    // rows of the longest segment
+  int q_tiles_max = 0;  // kWalkM-row tiles of the longest segment
 };
 
 struct ringattn_plan {
@@ -269,7 +268,7 @@ void fill_geometry(ringattn::BlockArgs& a, const ringattn_params& p, const Deriv
   a.half_partials = half_partials(p) ? 1 : 0;
 }
 
-inline int q_tiles_of(int len) { return (len + ringattn::kBlockM - 1) / ringattn::kBlockM; }
+inline int q_tiles_of(int len) { return (len + ringattn::kWalkM - 1) / ringattn::kWalkM; }
 
 // Appends one segment with its items to the tables.  part_base(i) / stride: where item i's
 // partial block lives.  A masked (diagonal) item runs last and the q tiles go busiest first.
@@ -303,7 +302,6 @@ void push_segment(ringattn_plan* pl, TableSlice& slice, int q_start, int q_len,
   pl->h_segs.push_back(sg);
   ++slice.seg_count;
   slice.q_tiles_max = std::max(slice.q_tiles_max, q_tiles_of(q_len));
-  slice.max_q_len = std::max(slice.max_q_len, q_len);
 }
 
 // The tables of a plan (host side; nothing here touches the GPU).
@@ -431,13 +429,8 @@ int launch_slice(const ringattn_plan* pl, const TableSlice& sl, ringattn::BlockA
   a.segs = pl->d_segs + sl.seg_begin;
   a.items = pl->d_segitems;
   a.n_segs = sl.seg_count;
-  if (a.mode == ringattn::kBlockCarryState) {  // no partials to emit: the two-phase kernel on 256-row tiles
-    a.q_tiles_max = (sl.max_q_len + ringattn::kWalkM - 1) / ringattn::kWalkM;
-    RA_HIP(ringattn::launch_walk(a, pl->p.dtype, pl->p.dim, stream));
-    return RINGATTN_OK;
-  }
   a.q_tiles_max = sl.q_tiles_max;
-  RA_HIP(ringattn::launch_block(a, pl->p.dtype, pl->p.dim, stream));
+  RA_HIP(ringattn::launch_walk(a, pl->p.dtype, pl->p.dim, stream));
   return RINGATTN_OK;
 }
 
@@ -566,7 +559,7 @@ int run_rank_call(const RankCall& rc, void* scratch, const void* q, const void* 
   a.segs = d_seg;
   a.items = d_items;
   a.n_segs = 1;
-  a.q_tiles_max = (c + ringattn::kWalkM - 1) / ringattn::kWalkM;
+  a.q_tiles_max = q_tiles_of(c);
   a.bh_stride = (int64_t)c * dim;  // q and out hold this rank's rows only; k and v the whole sequence
   a.S = c;
   RA_HIP(ringattn::launch_walk(a, rc.p.dtype, dim, stream));

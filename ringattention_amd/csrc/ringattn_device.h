@@ -108,4 +108,186 @@ static __device__ __forceinline__ bool decode_job(const BlockArgs& a, Segment& s
   return true;
 }
 
+// ---- conversions of 8 columns of a row, shared by the merge kernel and the merge at the end of a workgroup
+template <int DT> struct Store8;
+template <> struct Store8<0> {
+  static __device__ __forceinline__ void st(void* p, const float* x) {
+    f16x8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (_Float16)x[e];
+    *(f16x8*)p = v;
+  }
+};
+template <> struct Store8<1> {
+  static __device__ __forceinline__ void st(void* p, const float* x) {
+    bf16x8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (__bf16)x[e];
+    *(bf16x8*)p = v;
+  }
+};
+
+// 8 consecutive columns of one partial row as floats
+template <bool HP> struct PartRow;
+template <> struct PartRow<false> {
+  using ptr = const float*;
+  static __device__ __forceinline__ void ld(ptr p, f32x4& x0, f32x4& x1) {
+    x0 = *(const f32x4*)p;
+    x1 = *(const f32x4*)(p + 4);
+  }
+};
+template <> struct PartRow<true> {
+  using ptr = const _Float16*;
+  static __device__ __forceinline__ void ld(ptr p, f32x4& x0, f32x4& x1) {
+    const f16x8 v = *(const f16x8*)p;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      x0[e] = (float)v[e];
+      x1[e] = (float)v[4 + e];
+    }
+  }
+};
+
+// ---- merge of one job's rows (BM rows of a segment, one head) over the partials of the
+// segment's items.  The same arithmetic, in the same order, as merge_row; only the loads are
+// arranged differently: the block kernel, which runs this at the end of a workgroup, has just two
+// waves per SIMD to hide memory latency with, and every round trip it waits for is time its
+// compute unit runs half empty.  So all partial LSEs are fetched in one sweep and parked in LDS
+// (lse_s: [items][128] floats), and the partial O rows move in batches of 256 bytes per thread
+// (two output rows x four or eight parts), three batches in flight at any time.
+typedef __attribute__((address_space(3))) float lds_float;
+template <int DT, int D, bool HP, int BM, int THREADS>
+static __device__ __forceinline__ void merge_job_rows(const void* o_part, const float* lse_part, void* out, float* lse,
+                                                      const SegItem* items, const Segment& seg, int bh, int qt, int S,
+                                                      lds_float* lse_s) {
+  constexpr int WAVES = THREADS / 64;
+  constexpr int TPR = D / 8;  // threads per row, 8 columns each
+  constexpr int ROWS = THREADS / TPR;
+  constexpr int R = 2, G = HP ? 8 : 4;  // rows per thread and parts per batch: 64 registers a batch
+  constexpr int RSTEP = R * ROWS;
+  constexpr int KMAX = kMaxParts / WAVES;  // parts per wave in the LSE sweep
+  constexpr int LR = BM / 64;              // rows per lane in the LSE sweep
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n_parts = seg.item_count;
+  const SegItem* its = items + seg.item_begin;
+  const int row0 = qt * BM;  // first row of the job within the segment
+  __syncthreads();  // the partial stores of all waves have completed and are visible to them; the LDS is idle
+  {
+    float v[KMAX][LR];
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      const int i = wave + WAVES * k;
+      if (i < n_parts) {
+        const int64_t prow = its[i].part_base + (int64_t)bh * its[i].part_bh_stride + row0;
+#pragma unroll
+        for (int r = 0; r < LR; ++r) v[k][r] = (row0 + lane + 64 * r < seg.q_len) ? lse_part[prow + lane + 64 * r] : -INFINITY;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      const int i = wave + WAVES * k;
+      if (i < n_parts) {
+#pragma unroll
+        for (int r = 0; r < LR; ++r) lse_s[i * BM + lane + 64 * r] = v[k][r];
+      }
+    }
+  }
+  __syncthreads();
+  const int c8 = tid % TPR, rsub = tid / TPR;
+  // this thread's 8 columns of a partial row: 16 bytes as fp16, 32 as fp32
+  constexpr int PB = HP ? 16 : 32;
+  constexpr int NV = PB / 16;
+  const char* o_base = (const char*)o_part + c8 * PB;
+  const int n_groups = (n_parts + G - 1) / G;
+  const int n_batches = (BM / RSTEP) * n_groups;  // batch b: rows of b / n_groups, parts of b % n_groups
+  struct Batch {
+    f32x4 raw[R][G][NV];  // as loaded; fp16 partials are widened when they are used
+  };
+  auto row_of = [&](int b, int j) { return (b / n_groups) * RSTEP + j * ROWS + rsub; };  // within the job
+  auto fetch = [&](int b, Batch& t) {
+    const int i0 = (b % n_groups) * G;
+#pragma unroll
+    for (int u = 0; u < G; ++u)
+      if (i0 + u < n_parts) {
+        const int64_t prow = its[i0 + u].part_base + (int64_t)bh * its[i0 + u].part_bh_stride + row0;
+#pragma unroll
+        for (int j = 0; j < R; ++j)
+          if (row0 + row_of(b, j) < seg.q_len) {
+            const char* src = o_base + (prow + row_of(b, j)) * (D * (PB / 8));
+#pragma unroll
+            for (int v = 0; v < NV; ++v) t.raw[j][u][v] = *(const f32x4*)(src + 16 * v);
+          }
+      }
+  };
+  float mx[R], wsum[R], acc[R][8];
+  auto accumulate = [&](int b, const Batch& t) {
+    const int g = b % n_groups, i0 = g * G;
+    if (g == 0) {  // new rows: L = max over the parts first
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        mx[j] = -INFINITY;
+        wsum[j] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
+      }
+      for (int i = 0; i < n_parts; ++i)
+#pragma unroll
+        for (int j = 0; j < R; ++j) mx[j] = fmaxf(mx[j], lse_s[i * BM + row_of(b, j)]);
+    }
+#pragma unroll
+    for (int u = 0; u < G; ++u)
+      if (i0 + u < n_parts) {
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          const float L = lse_s[(i0 + u) * BM + row_of(b, j)];
+          if (row0 + row_of(b, j) >= seg.q_len || L == -INFINITY) continue;  // identity element: its O may hold anything
+          const float w = __expf(L - mx[j]);
+          wsum[j] += w;
+          float x[8];
+          if (HP) {
+            const f16x8 hv = __builtin_bit_cast(f16x8, t.raw[j][u][0]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = (float)hv[e];
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              x[e] = t.raw[j][u][0][e];
+              x[4 + e] = t.raw[j][u][NV - 1][e];
+            }
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[j][e] = __builtin_fmaf(w, x[e], acc[j][e]);
+        }
+      }
+    if (g == n_groups - 1) {  // all parts in: normalise and store
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        if (row0 + row_of(b, j) >= seg.q_len) continue;
+        if (mx[j] != -INFINITY) {
+          const float inv = 1.f / wsum[j];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[j][e] *= inv;
+        }
+        const int64_t out_row = (int64_t)bh * S + seg.q_start + row0 + row_of(b, j);
+        Store8<DT>::st((char*)out + (out_row * D + c8 * 8) * 2, acc[j]);
+        if (c8 == 0) lse[out_row] = (mx[j] == -INFINITY) ? -INFINITY : mx[j] + __logf(wsum[j]);
+      }
+    }
+  };
+  // three batches in flight
+  Batch t0, t1, t2;
+  fetch(0, t0);
+  if (1 < n_batches) fetch(1, t1);
+#pragma unroll 1
+  for (int b = 0; b < n_batches; b += 3) {
+    if (b + 2 < n_batches) fetch(b + 2, t2);
+    accumulate(b, t0);
+    if (b + 3 < n_batches) fetch(b + 3, t0);
+    if (b + 1 < n_batches) accumulate(b + 1, t1);
+    if (b + 4 < n_batches) fetch(b + 4, t1);
+    if (b + 2 < n_batches) accumulate(b + 2, t2);
+  }
+}
+
 }  // namespace ringattn

@@ -6,7 +6,6 @@
 
 namespace ringattn {
 
-constexpr int kBlockM = 128;  // query rows per workgroup of block_attention_kernel (4 waves x 32 rows)
 constexpr int kWalkM = 256;   // query rows per workgroup of ring_walk_kernel (8 waves x 32 rows)
 constexpr int kMaxParts = 64; // partial slots a merge can combine
 
@@ -29,7 +28,7 @@ struct WorkItem {
 
 // What the block kernel runs: a SEGMENT is a range of query rows (of every head) together with
 // ALL the key ranges it meets -- the ring steps of the reference's step loop
-// (csrc/ring_attention.cu:456-620) for those rows.  One workgroup owns 128 rows of a segment,
+// (csrc/ring_attention.cu:456-620) for those rows.  One workgroup owns kWalkM rows of a segment,
 // keeps their Q in registers and walks the segment's items, as the reference's CTA walks the
 // ring steps (:439-443,456), emitting one (partial O, partial LSE) per item.
 struct SegItem {
@@ -55,10 +54,10 @@ static_assert(sizeof(Segment) == 32, "Segment is read as two 16-byte scalar load
 
 // What a workgroup does with the softmax state (max, sum, acc-O) of its rows between the KV chunks it walks.
 enum BlockMode {
-  kBlockPartials = 0,        // per chunk: emit the normalised partial (O, LSE), reset the state   (launch_block)
-  kBlockPartialsMerged = 1,  // the same, and after the last chunk merge the partials of the rows into out / lse   (launch_block)
+  kBlockPartials = 0,        // per chunk: emit the normalised partial (O, LSE), reset the state
+  kBlockPartialsMerged = 1,  // the same, and after the last chunk merge the partials of the rows into out / lse
   kBlockCarryState = 2,      // carry the state across the chunks, as the reference's CTA does across its ring
-                             // steps (csrc/ring_attention.cu:439-443,597), and write out / lse once: no partials   (launch_walk)
+                             // steps (csrc/ring_attention.cu:439-443,597), and write out / lse once: no partials
 };
 
 struct BlockArgs {
@@ -77,7 +76,7 @@ struct BlockArgs {
   int64_t bh_stride;   // elements between heads of q and out (= S * D)
   int64_t kv_bh_stride;      // elements between heads of k and v
   int S;               // rows per head of q, out and lse
-  int q_tiles_max;     // q tiles (kBlockM rows; kWalkM for launch_walk) of the longest segment (grid dimension)
+  int q_tiles_max;     // kWalkM-row q tiles of the longest segment (grid dimension)
   int n_segs;
   int BH;              // batch * heads
   int heads;           // query heads per batch entry
@@ -119,9 +118,7 @@ struct TablePack {
 };
 
 // dtype: 0 = fp16, 1 = bf16.  Return hipSuccess or the launch error.
-hipError_t launch_block(const BlockArgs& a, int dtype, int dim, hipStream_t stream);
-// the same work in kBlockCarryState mode by ring_walk_kernel (ringattn_walk.hip): 256-row q tiles, two-phase blocks
-hipError_t launch_walk(const BlockArgs& a, int dtype, int dim, hipStream_t stream);
+hipError_t launch_walk(const BlockArgs& a, int dtype, int dim, hipStream_t stream);  // ring_walk_kernel, any BlockMode
 hipError_t launch_merge(const MergeArgs& a, int dtype, int dim, hipStream_t stream);
 // writes pack.seg to *seg_dst and pack.items[0..n) to item_dst
 hipError_t launch_write_table(const TablePack& pack, int n, Segment* seg_dst, SegItem* item_dst, hipStream_t stream);

@@ -1,16 +1,40 @@
-// gfx950 (CDNA4) kernel: the ring-attention forward with the softmax state carried through the
-// ring steps, in its two-phase form.
+// gfx950 (CDNA4) kernel: block attention over the ring steps of 256 query rows.
 //
 //   ring_walk_kernel : a workgroup of EIGHT waves owns 256 query rows of a segment (one head),
-//       keeps their Q in registers and walks the KV chunks those rows meet with the running max,
-//       sum and acc-O in registers from the first chunk to the last, as the reference's CTA does
-//       across its ring steps (csrc/ring_attention.cu:439-443,456,597); O = acc / l
-//       (:621-664) and LSE are written once.  The arithmetic per tile is that of
-//       block_attention_kernel (ringattn_kernels.hip): S^T = K Q^T and O^T += V^T P^T on
-//       v_mfma_f32_32x32x16, online softmax with a lazy reference max, K/V tiles through two
-//       4-deep LDS rings filled by direct-to-LDS loads, one barrier per two tiles.
+//       keeps their Q in registers and walks the KV chunks those rows meet, as the reference's
+//       CTA walks its ring steps (csrc/ring_attention.cu:439-443,456), per chunk
+//       S^T = K Q^T, online softmax with running max / sum, O^T += V^T P^T.
+//       Between two chunks it either carries max, sum and acc-O on (the reference's own way,
+//       :597, with O = acc / l (:621-664) and the LSE written once at the end), or emits the
+//       chunk's normalised partial (O, LSE) and starts afresh (the ring steps kept apart; the
+//       partials of its rows can then be merged at the end of the workgroup).
+//       It restates the inner KV-tile loop of the reference kernel
+//       (csrc/ring_attention.cu:536-610: gemm_smem :278-301, softmax_rescale_o
+//       :194-245 completed with the missing `sum += sum_cur` tail,
+//       scale_apply_exp2 :173-192, gemm_A_in_regs :304-324) and its epilogue
+//       (:621-664), with the tiling of csrc/kernel_traits.h:11-177 replaced by a
+//       wave64 / MFMA 32x32x16 design:
+//         * each of the 8 waves owns 32 query rows; Q lives in registers as the
+//           B operand for the whole launch (the reference re-reads it from smem
+//           for every tile, :565);
+//         * the score tile is computed TRANSPOSED (keys x queries), so one lane
+//           holds 16 keys of ONE query: row max / row sum are in-register
+//           reductions plus one cross-half exchange, and the probabilities are
+//           already in B-operand layout for O^T += V^T P^T -- the MFMA analogue
+//           of convert_layout_rowcol_Aregs (:260-276);
+//         * K and V go HBM -> LDS directly (global_load_lds_dwordx4) in 32-key
+//           tiles, through two 4-deep rings, one barrier per two tiles; bank
+//           conflicts are removed by an XOR swizzle applied on the
+//           global-address side;
+//         * V^T operands come from ds_read_b64_tr_b16 (the LDS transpose read),
+//           replacing ldmatrix.trans of csrc/kernel_traits.h:39;
+//         * the exponent offset m is a REFERENCE max: it is moved (with the rescale of l and
+//           acc-O of :226-232) only when some row's tile max exceeds it by more than
+//           2^kLazyLog2, decided by a wave-uniform branch.  Until then p = exp2((s - m) k2)
+//           may exceed 1 (by at most 2^kLazyLog2, well inside fp16 and bf16 range); O = acc / l
+//           and LSE = (m k2 + log2 l) ln 2 do not depend on the choice of m.
 //
-//       What differs is how a tile's work is laid out in time.  The eight waves sit two per SIMD
+//       A tile's work is laid out in time in two phases.  The eight waves sit two per SIMD
 //       (wave w and wave w + 4).  Per tile every wave has an MFMA phase (O^T += V(u)^T P(u)^T, then
 //       S^T(u+1) = K(u+1) Q^T: 16 MFMAs and their 24 fragment reads from LDS at d = 128) and a
 //       softmax phase (row max, reference move, exponentials, row sum, conversion of P: VALU
@@ -18,14 +42,19 @@
 //       phase, between the same barriers: while one wave of a SIMD keeps the matrix pipe busy the
 //       other keeps the VALU busy, instead of both mixing the two kinds of work and colliding.
 //       Measured on synthetic tiles (same instruction mix, barrier and loads): 63.6 % of the
-//       MFMA-only rate against 53.4 % for the mixed stream.
+//       MFMA-only rate against 53.4 % for a stream that mixes both kinds of work in every wave.
+//
+//       From one KV chunk to the next the tile pipeline keeps running where the shapes allow it
+//       (the loads that run ahead of the last tiles fetch the first tiles of the next chunk).
 #include "ringattn_device.h"
 
 #include <type_traits>
 
 namespace ringattn {
 
-template <int DT, int D>
+// KEEP: the softmax state is carried through the chunks (kBlockCarryState); otherwise a partial is emitted per
+// chunk (kBlockPartials, kBlockPartialsMerged; HP: partial O as fp16).
+template <int DT, int D, bool HP, bool KEEP>
 __global__ __launch_bounds__(512, 1) void ring_walk_kernel(const BlockArgs a) {
   using E = Elem<DT>;
   constexpr int WAVES = 8;
@@ -41,7 +70,9 @@ __global__ __launch_bounds__(512, 1) void ring_walk_kernel(const BlockArgs a) {
   constexpr float kLazyLog2 = 8.f;
   static_assert(BM == 32 * WAVES, "one 32-row block per wave");
   static_assert(PIECES == WAVES || 2 * PIECES == WAVES, "a tile is loaded by all waves, or K and V by half of them each");
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * NBUF * TILE];  // K ring, V ring
+  // K ring, V ring; at the end of a workgroup that merges its partials, their LSEs ([parts][256] floats)
+  constexpr int kRingBytes = 2 * NBUF * TILE, kLseBytes = KEEP ? 0 : kMaxParts * BM * (int)sizeof(float);
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[kRingBytes > kLseBytes ? kRingBytes : kLseBytes];
 
   const unsigned smem_base = lds_offset(smem);
   const int tid = threadIdx.x, lane = tid & 63;
@@ -107,6 +138,16 @@ __global__ __launch_bounds__(512, 1) void ring_walk_kernel(const BlockArgs a) {
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
+  auto reset_state = [&]() {
+    m = -INFINITY;
+    ms = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ls[i] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
+  };
   f32x16 sacc;   // scores of the tile in flight: written by an MFMA phase, consumed by the next softmax phase
   s16x8 pf[2];   // its probabilities in B-operand layout: written by a softmax phase, consumed by the next MFMA phase
 
@@ -260,10 +301,45 @@ __global__ __launch_bounds__(512, 1) void ring_walk_kernel(const BlockArgs a) {
 #pragma unroll
     for (int i = 0; i < KS; ++i) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
   };
+  // Set between a carried-over chunk boundary and the first pair of the next chunk when a partial is stored
+  // in between: the tiles that pair needs were waited for (and the barrier passed) BEFORE the stores, so that
+  // the pair does not wait for them (stores count in vmcnt too).
+  bool synced = false;
   auto ring_barrier = [&]() {
+    if (synced) {
+      synced = false;
+      return;
+    }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   };
+  // a chunk's partial (csrc/ring_attention.cu:621-633): normalise, emit O and LSE
+  auto emit_partial = [&](const SegItem* w) {
+    const float l = cross_half_sum((ls[0] + ls[1]) + (ls[2] + ls[3]));
+    const float inv = (l > 0.f) ? 1.f / l : 0.f;
+    const int row_l = qt * BM + 32 * wave + n;
+    if (row_l >= q_len) return;  // a row beyond the query range
+    const int64_t prow = w->part_base + (int64_t)bh * w->part_bh_stride + row_l;
+    const int64_t opos = prow * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 val;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) val[e] = oacc[db][4 * q4 + e] * inv;
+        if (HP) {  // fp16 partials: |O_part| <= max |V|, the caller vouches that this fits
+          f16x4 hv;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) hv[e] = (_Float16)val[e];
+          *(f16x4*)((_Float16*)a.o_part + opos + 32 * db + 8 * q4 + 4 * h) = hv;
+        } else {
+          *(f32x4*)((float*)a.o_part + opos + 32 * db + 8 * q4 + 4 * h) = val;
+        }
+      }
+    if (h == 0) a.lse_part[prow] = (l > 0.f) ? (ms + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
+  };
+  constexpr bool keep_state = KEEP;
 
   // The walk of all items, for one half of the workgroup.  At the start of block u the waves of the
   // first half hold P(u) (their softmax phase of tile u is done), those of the second half the raw
@@ -398,16 +474,31 @@ __global__ __launch_bounds__(512, 1) void ring_walk_kernel(const BlockArgs a) {
         block(C3{}, std::true_type{}, std::true_type{}, u + 3);
       }
       for (; u < n_tiles; ++u) block(C0{}, std::false_type{}, std::false_type{}, u);
-      if (!carry) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // re-reads of the last tile
       carried = carry;
+      if (keep_state) {
+        // the softmax state runs on into the next chunk; with the pipeline carried over as well, the chunk
+        // boundary is just another tile boundary
+        if (!carry) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // re-reads of the last tile
+        continue;
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next chunk's first tiles, or re-reads of the last tile
+      if (carry) {
+        __syncthreads();
+        synced = true;
+      }
+      emit_partial(w);
+      reset_state();
     }
   };
   if (wave < WAVES / 2) walk(std::false_type{});
   else walk(std::true_type{});
 
-  // the rows' result: the reference's epilogue (csrc/ring_attention.cu:621-664), O = acc / l in the
-  // storage type, plus the LSE
-  {
+  if (!KEEP && a.mode == kBlockPartialsMerged)  // this workgroup's rows over the partials it has just written
+    merge_job_rows<DT, D, HP, BM, 64 * WAVES>(a.o_part, a.lse_part, a.out, a.lse, a.items, seg, bh, qt, a.S,
+                                              (lds_float*)(__attribute__((address_space(3))) void*)smem);
+  // the rows' result from a carried state: the reference's epilogue (csrc/ring_attention.cu:621-664), O = acc / l
+  // in the storage type, plus the LSE
+  if (keep_state) {
     const float l = cross_half_sum((ls[0] + ls[1]) + (ls[2] + ls[3]));
     const float inv = (l > 0.f) ? 1.f / l : 0.f;
     const int row_l = qt * BM + 32 * wave + n;
@@ -430,16 +521,23 @@ __global__ __launch_bounds__(512, 1) void ring_walk_kernel(const BlockArgs a) {
 
 hipError_t launch_walk(const BlockArgs& a, int dtype, int dim, hipStream_t stream) {
   if (a.n_segs <= 0) return hipSuccess;
-  if (a.mode != kBlockCarryState) return hipErrorInvalidValue;
   const int q_tiles = a.q_tiles_max;  // kWalkM-row tiles of the longest segment
   const int64_t groups = (int64_t)a.n_segs * a.BH;
   const int64_t blocks = (a.groups ? (int64_t)a.groups_per_xcd : (groups + 7) / 8) * 8 * q_tiles;
   if (q_tiles <= 0 || blocks > INT32_MAX) return hipErrorInvalidValue;
   const unsigned grid = (unsigned)blocks;
-  if (dtype == 0 && dim == 64) ring_walk_kernel<0, 64><<<grid, 512, 0, stream>>>(a);
-  else if (dtype == 0 && dim == 128) ring_walk_kernel<0, 128><<<grid, 512, 0, stream>>>(a);
-  else if (dtype == 1 && dim == 64) ring_walk_kernel<1, 64><<<grid, 512, 0, stream>>>(a);
-  else if (dtype == 1 && dim == 128) ring_walk_kernel<1, 128><<<grid, 512, 0, stream>>>(a);
+  if (a.mode != kBlockCarryState && a.mode != kBlockPartials && a.mode != kBlockPartialsMerged) return hipErrorInvalidValue;
+#define RA_LAUNCH_WALK(DT_, D_)                                                                          \
+  do {                                                                                                \
+    if (a.mode == kBlockCarryState) ring_walk_kernel<DT_, D_, false, true><<<grid, 512, 0, stream>>>(a);   \
+    else if (a.half_partials) ring_walk_kernel<DT_, D_, true, false><<<grid, 512, 0, stream>>>(a);         \
+    else ring_walk_kernel<DT_, D_, false, false><<<grid, 512, 0, stream>>>(a);                             \
+  } while (0)
+  if (dtype == 0 && dim == 64) RA_LAUNCH_WALK(0, 64);
+  else if (dtype == 0 && dim == 128) RA_LAUNCH_WALK(0, 128);
+  else if (dtype == 1 && dim == 64) RA_LAUNCH_WALK(1, 64);
+  else if (dtype == 1 && dim == 128) RA_LAUNCH_WALK(1, 128);
+#undef RA_LAUNCH_WALK
   else return hipErrorInvalidValue;
   return hipGetLastError();
 }

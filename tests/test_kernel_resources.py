@@ -1,9 +1,7 @@
-"""What the compiler made of the attention kernels: the d = 128 instantiations must keep two
-waves per SIMD (256 registers) and their steady key loops -- the loops that hold 64 MFMAs, four
-32-key blocks -- must not touch scratch memory.  (block_attention_kernel as a whole does spill a
-few values around the chunk prologue and the general, non-unrolled blocks; those run once per
-chunk.  ring_walk_kernel must not spill at all.)
-Compiles the kernels to assembly for gfx950; needs hipcc but no GPU."""
+"""What the compiler made of the attention kernel: every instantiation must fit two waves per
+SIMD (256 registers) without scratch memory, and the steady key loops of the d = 128 ones -- the
+loops that hold 64 MFMAs, four 32-key blocks -- must carry one barrier per two tiles.
+Compiles the kernel to assembly for gfx950; needs hipcc but no GPU."""
 import os
 import re
 import shutil
@@ -78,34 +76,19 @@ def steady_loops(asm, kernel):
 def test_walk_kernel_runs_two_waves_per_simd_without_spills(tmp_path):
     asm, usage = compile_to_asm("ringattn_walk.hip", tmp_path / "walk.s")
     walks = {n: u for n, u in usage.items() if "ring_walk_kernel" in n}
-    assert len(walks) == 4                                     # {fp16, bf16} x {64, 128}
+    # {fp16, bf16} x {64, 128} x {carried state; partials as fp32; partials as fp16}
+    assert len(walks) == 12
     for n, u in walks.items():
+        carried = n.endswith("Lb0ELb1EEEvNS_9BlockArgsE")
         assert u["ScratchSize [bytes/lane]"] == 0, (n, u)
         assert u["VGPRs"] <= 256, (n, u)                       # eight waves per workgroup, one workgroup per compute unit
-        assert u["LDS Size [bytes/block]"] == (65536 if "Li128E" in n else 32768), (n, u)
+        # K and V rings; the variants that merge park the partial LSEs of their 256 rows there afterwards
+        assert u["LDS Size [bytes/block]"] == (32768 if carried and "Li64E" in n else 65536), (n, u)
         if "Li128E" in n:
             steady = steady_loops(asm, n)
             assert len(steady) == 4, (n, len(steady))          # plain and masked groups, for each half of the workgroup
             for lab, ins in steady:
-                assert sum(i.startswith("s_barrier") for i in ins) == 2, (n, lab)   # one barrier per two tiles
-
-
-def test_steady_key_loops_are_spill_free_at_two_waves_per_simd(tmp_path):
-    asm, usage = compile_to_asm("ringattn_kernels.hip", tmp_path / "kernels.s")
-    blocks = {n: u for n, u in usage.items() if "block_attention_kernel" in n}
-    assert len(blocks) == 8                                    # {fp16, bf16} x {64, 128} x {fp32, fp16 partials}
-    for n, u in blocks.items():
-        assert u["Occupancy [waves/SIMD]"] == 2, (n, u)
-        assert u["VGPRs"] <= 256, (n, u)
-        if "Li128E" in n:
-            assert u["LDS Size [bytes/block]"] == 65536, (n, u)   # two workgroups per compute unit
-    checked = 0
-    for n in blocks:
-        if "Li128E" not in n:
-            continue
-        steady = steady_loops(asm, n)
-        assert len(steady) == 2, (n, len(steady))              # the plain and the masked groups of four blocks
-        for lab, ins in steady:
-            assert not any(i.startswith("scratch_") for i in ins), (n, lab)
-            checked += 1
-    assert checked == 8
+                # one barrier per two tiles (where partials are emitted the first one of a chunk may have been
+                # taken before the stores, which puts it on a side path of the loop)
+                assert sum(i.startswith("s_barrier") for i in ins) in ((2,) if carried else (1, 2)), (n, lab)
+                assert not any(i.startswith("scratch_") for i in ins), (n, lab)
