@@ -32,10 +32,10 @@ PEAK_HBM_GBS = 8000.0
 # (bytes, summary under profiles/, kernel_source_id() when it was measured).  The figure is only printed while the
 # kernel source is still the one that was profiled.
 MEASURED_TRAFFIC = {
-    "cfg4": (3404e6, "profiles/ring_walk_kernel_cfg4.md", "b72efe25495fa5c4"),
-    "cfg2": (34.1e6, "profiles/ring_walk_kernel_other_workloads.md", "b72efe25495fa5c4"),
-    "cfg3": (2217e6, "profiles/ring_walk_kernel_other_workloads.md", "b72efe25495fa5c4"),
-    "cfg5": (18260e6, "profiles/ring_walk_kernel_other_workloads.md", "b72efe25495fa5c4"),
+    "cfg4": (3489e6, "profiles/ring_walk_kernel_cfg4.md", "2a6f50c5975f4ba6"),
+    "cfg2": (34.1e6, "profiles/ring_walk_kernel_other_workloads.md", "2a6f50c5975f4ba6"),
+    "cfg3": (2209e6, "profiles/ring_walk_kernel_other_workloads.md", "2a6f50c5975f4ba6"),
+    "cfg5": (18260e6, "profiles/ring_walk_kernel_other_workloads.md", "2a6f50c5975f4ba6"),
 }
 BASELINE_METRIC = "ring-attn fwd TFLOP/s + % bf16 MFMA peak, S=32K d=128 8-step ring, 1 GPU"
 
@@ -127,7 +127,7 @@ def main():
 
     bh = w.batch * w.heads
     peak = PEAK_TFLOPS[w.dtype]
-    # ---- block kernel: the same forward on a plan that records an event pair around its
+    # ---- attention kernel: the same forward on a plan that records an event pair around its
     # block-attention launch, on the stream it is launched on.  The launch is the whole ring (every
     # step of every rank).
     timed = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=False,

@@ -51,7 +51,7 @@ extern "C" {
 #define RINGATTN_FLAG_TIMING 2     /* record timing events around every block-attention launch of ringattn_fwd
                                       (read with ringattn_plan_launch_times); ignored together with FLAG_GRAPH */
 #define RINGATTN_FLAG_HALF_PARTIALS 4 /* keep the per-step partial O in fp16 instead of fp32 (for either input dtype): halves
-                                      the workspace and the bytes the block kernel writes and the merge reads.  A partial O
+                                      the workspace and the bytes the attention kernel writes and the merge reads.  A partial O
                                       row is a weighted mean of V rows, so this needs |V| < 65504, and it adds up to 2^-11
                                       relative error per partial (fp32 partials add none); the partial LSE stays fp32.
                                       Applies wherever partials are written (ringattn_block_fwd, ringattn_rank_step_fwd,
@@ -256,8 +256,8 @@ int ringattn_ring_attention(const void* q, const void* k, const void* v, void* o
  * reference (whose entry allocates on every call, csrc/ring_attention.cu:383-394).  Same
  * arguments and results as ringattn_ring_attention, plus the stream; it calls no hipMalloc,
  * hipFree, memcpy or other allocating routine and does not synchronise: the work (a
- * table-writing kernel, then the block kernel) is queued on `stream`.  The table of ring steps
- * the block kernel reads (32 bytes + 32 per visible step), which ringattn_ring_attention keeps
+ * table-writing kernel, then the attention kernel) is queued on `stream`.  The table of ring steps
+ * the attention kernel reads (32 bytes + 32 per visible step), which ringattn_ring_attention keeps
  * in a per-call allocation, lives in a static device array of ringattn_noalloc_scratch_bytes()
  * bytes (4 KiB, held by every GPU the library runs on until the process ends): enough for
  * RINGATTN_MAX_NPES steps, and a ring with more ranks is refused with RINGATTN_ERR_NPES like

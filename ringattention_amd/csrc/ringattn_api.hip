@@ -132,7 +132,7 @@ void append_items(std::vector<ringattn::WorkItem>& out, const Derived& d, int P,
 }
 
 // A SEGMENT: rows of one rank that meet the same ring steps, with those steps' key ranges in
-// ascending step order -- what one workgroup of the block kernel walks (the reference's CTA
+// ascending step order -- what one workgroup of the attention kernel walks (the reference's CTA
 // walks the steps of its rows the same way, csrc/ring_attention.cu:456-620).  Contiguous
 // layouts have one segment per rank; a zigzag rank has two (its low half sees fewer steps).
 struct HostSegment {
@@ -172,7 +172,7 @@ void rank_segments(std::vector<HostSegment>& out, const Derived& d, int P, bool 
   }
 }
 
-// All segments of a forward, busiest first: the block kernel's workgroups are dispatched in
+// All segments of a forward, busiest first: the attention kernel's workgroups are dispatched in
 // this order, so the launch ends on its shortest ones.
 std::vector<HostSegment> forward_segments(const Derived& d, int P, bool causal) {
   std::vector<HostSegment> segs;
@@ -435,7 +435,7 @@ int launch_slice(const ringattn_plan* pl, const TableSlice& sl, ringattn::BlockA
 }
 
 // The ring step loop (csrc/ring_attention.cu:456-620) and the epilogue (:621-664), ONE launch:
-// every workgroup walks the ring steps of its 128 rows with the softmax state carried in
+// every workgroup walks the ring steps of its 256 rows with the softmax state carried in
 // registers, like the reference's CTA (:439-443,597).  With RINGATTN_FLAG_STEP_PARTIALS it
 // writes a partial (O, LSE) per step instead and merges them at the end.
 int run_forward(ringattn_plan* pl, const void* q, const void* k, const void* v, void* out,
@@ -478,7 +478,7 @@ inline bool plan_ok(const ringattn_plan* pl) {
 
 // ---- the reference-shaped call for one rank (ringattn_ring_attention and its variant that
 // allocates nothing) ------------------------------------------------------------------------
-// Device scratch of one call: the segment + item table the block kernel reads (the softmax state
+// Device scratch of one call: the segment + item table the attention kernel reads (the softmax state
 // is carried in registers across the ring steps, so there are no partials to park).
 struct RankCall {
   ringattn_params p;
@@ -539,7 +539,7 @@ int prepare_rank_call(RankCall* rc, const void* q, const void* k, const void* v,
   return RINGATTN_OK;
 }
 
-// The table (written by a kernel from its arguments), then the block kernel: two launches on
+// The table (written by a kernel from its arguments), then the attention kernel: two launches on
 // `stream`, nothing is allocated or copied from the host.
 // `scratch`: rc.scratch_bytes of device memory, 32-byte aligned.
 int run_rank_call(const RankCall& rc, void* scratch, const void* q, const void* k, const void* v, void* out,

@@ -150,7 +150,7 @@ template <> struct PartRow<true> {
 
 // ---- merge of one job's rows (BM rows of a segment, one head) over the partials of the
 // segment's items.  The same arithmetic, in the same order, as merge_row; only the loads are
-// arranged differently: the block kernel, which runs this at the end of a workgroup, has just two
+// arranged differently: the attention kernel, which runs this at the end of a workgroup, has just two
 // waves per SIMD to hide memory latency with, and every round trip it waits for is time its
 // compute unit runs half empty.  So all partial LSEs are fetched in one sweep and parked in LDS
 // (lse_s: [items][128] floats), and the partial O rows move in batches of 256 bytes per thread

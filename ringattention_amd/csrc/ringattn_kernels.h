@@ -26,7 +26,7 @@ struct WorkItem {
   int pad0, pad1;
 };
 
-// What the block kernel runs: a SEGMENT is a range of query rows (of every head) together with
+// What the attention kernel runs: a SEGMENT is a range of query rows (of every head) together with
 // ALL the key ranges it meets -- the ring steps of the reference's step loop
 // (csrc/ring_attention.cu:456-620) for those rows.  One workgroup owns kWalkM rows of a segment,
 // keeps their Q in registers and walks the segment's items, as the reference's CTA walks the

@@ -13,7 +13,7 @@
 
 namespace ringattn {
 
-// ---- merge of one row: shared by the merge kernel and the block kernel's fused merge -------
+// ---- merge of one row: the merge kernel's arithmetic (the attention kernel's merge at the end of a workgroup follows it) -------
 // The parts of one row, in ascending slot order: the set bits of a mask over equally spaced slots.
 struct SlotParts {
   uint64_t rest;
