@@ -8,11 +8,11 @@ of its 256 query rows with the softmax state in registers and writes O and LSE a
 Prints one JSON line.  `value` is algorithmic TFLOP/s (4*B*H*d*visible (q,k) pairs per forward)
 over the wall time of K steps; `roofline` prices the block-attention launch of the same forward
 against the dense MFMA peak, timed by an event pair on the launch stream (a second pass of K
-forwards on a plan with the timing flag); with --both-forwards, `forward_with_step_partials` is
-the same forward on a plan that keeps the ring steps apart (a partial (O, LSE) per step, merged
-at the end of each workgroup; --step-partials makes that one the headline, and every
-block-attention launch of a run without --both-forwards is of the headline kind, so a kernel
-trace of the run averages one kind of launch); `merge` times the merge kernel alone, on
+forwards on a plan with the timing flag); `forward_with_step_partials` is the same forward on a
+plan that keeps the ring steps apart (a fp32 partial (O, LSE) per step in a workspace, merged at
+the end of each workgroup: another instantiation of the kernel, so a kernel trace keeps the two
+apart; --step-partials makes that one the headline, --one-forward skips the other one); `merge`
+times the merge kernel alone, on
 caller-held per-step partials, against HBM bandwidth; `cpu_baseline` is the CPU oracle timed on
 this host on a bounded sample of the same workload's rows.
 """
@@ -77,7 +77,8 @@ def main():
     ap.add_argument("--rank-local", action="store_true",
                     help="also time the ring rank by rank on rank-local buffers (one launch per rank and step)")
     ap.add_argument("--per-step", action="store_true", help="also time one block-attention launch per ring step")
-    ap.add_argument("--both-forwards", action="store_true", help="also time the forward of the other kind (see --step-partials)")
+    ap.add_argument("--one-forward", action="store_true",
+                    help="skip the forward of the other kind (see --step-partials), which is timed as well by default")
     ap.add_argument("--step-partials", action="store_true",
                     help="time the forward that keeps the ring steps apart (per-step partials in a workspace, merged at "
                          "the end) instead of the one that carries the softmax state through the steps")
@@ -160,7 +161,7 @@ def main():
 
     # ---- the other forward (steps kept apart unless --step-partials, which swaps the two)
     other_leg = None
-    if args.both_forwards:
+    if not args.one_forward:
         other = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=w.graph, layout=args.layout,
                                   half_partials=w.half_partials, step_partials=not args.step_partials)
         for _ in range(2):
