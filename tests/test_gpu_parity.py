@@ -229,11 +229,14 @@ def test_unequal_rank_lengths(oracle, seqlen, causal, d, dtype):
 @pytest.mark.parametrize("seqlen,causal,d,dtype,layout", [
     ((100, 333, 1, 77), False, 64, "fp16", "contiguous"),
     ((100, 333, 1, 77), True, 128, "bf16", "contiguous"),
-    ((513,), True, 128, "fp16", "contiguous"),           # one rank, one row into a fifth q tile
+    ((513,), True, 128, "fp16", "contiguous"),           # one rank, one row into a third q tile
     ((31, 33), True, 64, "bf16", "contiguous"),          # shorter than one key tile / one more than it
     ((1000, 24), False, 128, "bf16", "contiguous"),
     ((130, 70, 2, 258), True, 128, "bf16", "zigzag"),
     ((1, 1, 1), True, 64, "fp16", "contiguous"),
+    ((257, 1023, 769), True, 128, "bf16", "contiguous"),   # several 256-row q tiles per rank, each rank one row or one tile off
+    ((1026, 514), True, 64, "fp16", "zigzag"),             # d = 64: K and V tiles loaded by different halves of the workgroup
+    ((640, 384, 896), False, 64, "bf16", "contiguous"),    # whole key tiles, chunk lengths that are no multiples of four tiles
 ])
 def test_ragged_lengths(oracle, seqlen, causal, d, dtype, layout):
     # lengths that are no multiples of the 128-row q tile or the 32-key tile: the tail
