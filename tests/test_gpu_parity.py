@@ -67,6 +67,9 @@ def check_rows(oracle, w, q, k, v, out, lse, rows, scale=None, half_partials=Non
     what rounding the probabilities to the storage type allows (each p is off by at most half an ulp
     relative and O is a p-weighted mean of V rows: 2^-(mantissa+1) max|V|) plus half an ulp for the store;
     only rows whose few dominant keys carry large V entries that nearly cancel reach the second form.
+    With an explicit softmax scale above 1/sqrt(d) (none of the workloads has one) the softmax is peaked, O stays as
+    large as single V rows, and a bf16 result one ulp from the rounded oracle in [2, 4) is 1.1e-2 from the exact
+    value: the first bound is then widened by the same p-rounding term.
     LSE: relative error <= 1e-3."""
     o_ref, l_ref = oracle.attention_rows(q, k, v, w.dtype, causal=w.causal, rows=rows, scale=scale)
     idx = torch.from_numpy(rows).cuda()
@@ -75,6 +78,10 @@ def check_rows(oracle, w, q, k, v, out, lse, rows, scale=None, half_partials=Non
     assert np.isfinite(o_gpu).all() and np.isfinite(l_gpu).all()
     ulp = storage_ulp(o_ref, w.dtype)
     tol = np.maximum(O_TOL, 0.5 * ulp)
+    v_max = bits_to_float64(np.array([(np.ascontiguousarray(v).view(np.uint16) & 0x7FFF).max()], dtype=np.uint16), w.dtype)[0]
+    p_round = 2.0 ** -((10 if w.dtype == "fp16" else 7) + 1) * v_max
+    if scale is not None and scale > 1.0 / math.sqrt(w.dim):
+        tol = np.maximum(tol, p_round + 0.5 * ulp)
     err = np.abs(o_gpu - o_ref)
     err_o = err.max()
     err_l = (np.abs(l_gpu - l_ref) / np.maximum(np.abs(l_ref), 1e-3)).max()
@@ -92,8 +99,7 @@ def check_rows(oracle, w, q, k, v, out, lse, rows, scale=None, half_partials=Non
     assert (err <= tol).all(), f"{w.name}: max|dO| = {err_o:.3e}, worst excess {(err - tol).max():.3e}"
     # fp16 per-step partials (RINGATTN_FLAG_HALF_PARTIALS) round once more on the way: two units then
     ulps = 2 if (w.half_partials if half_partials is None else half_partials) else 1
-    v_max = bits_to_float64(np.array([(np.ascontiguousarray(v).view(np.uint16) & 0x7FFF).max()], dtype=np.uint16), w.dtype)[0]
-    p_rounding = 2.0 ** -((10 if w.dtype == "fp16" else 7) + 1) * v_max + 0.5 * storage_ulp(o_rounded, w.dtype)
+    p_rounding = p_round + 0.5 * storage_ulp(o_rounded, w.dtype)
     over = int((err_r > ulps * ulp_r).any(axis=1).sum())
     if over:
         print(f"parity {w.name}: {over} of {len(rows)} rows beyond {ulps} ulp of the rounded oracle "
