@@ -295,8 +295,8 @@ def ring_attention(q, k, v, out, npes, mype, seqlen, dim, max_seq, lse=None, cau
 
 def ring_attention_noalloc(q, k, v, out, npes, mype, seqlen, dim, max_seq, lse=None, causal=False, softmax_scale=0.0,
                            stream=None):
-    """ring_attention() through the entry point that allocates nothing (static device scratch);
-    asynchronous on `stream`.  Raises RingattnError (workspace) if the rank's partials do not fit."""
+    """ring_attention() through the entry point that allocates nothing (its table of ring steps lives in a
+    static device scratch); asynchronous on `stream`."""
     lib = _lib.load()
     _check_rank_call(q, k, v, out, lse, npes, mype, seqlen, dim)
     arr = (ctypes.c_int * len(seqlen))(*[int(x) for x in seqlen])

@@ -27,11 +27,12 @@ namespace {
   RA_CHECK_DEVICE(x);     \
   RA_CHECK_CONTIGUOUS(x)
 
-// A plan owns ONE workspace and is meant for one forward at a time, so the cache holds a plan
-// per (parameter set, device, STREAM): forwards on different streams never share partials, and
+// A plan is meant for one forward at a time (its tables, its timing events, and with
+// RINGATTN_FLAG_STEP_PARTIALS its workspace, are single), so the cache holds a plan per
+// (parameter set, device, STREAM): forwards on different streams never share one, and
 // forwards on one stream are ordered by the stream.  A per-plan mutex keeps two host threads
 // from enqueueing on the same plan at once.  The cache is bounded: beyond kMaxPlans the least
-// recently used plan that nobody is enqueueing on is destroyed (its workspace goes back to the
+// recently used plan that nobody is enqueueing on is destroyed (its device memory goes back to the
 // device); hipFree inside ringattn_plan_destroy waits for the work that still uses it.
 using PlanKey = std::tuple<int, void*, std::vector<int>, int, int, int, int, int, int, int, float>;
 struct Entry {

@@ -3,8 +3,8 @@
 The op follows the conventions the reference's include/attention_api.cuh:12-18 sets for a
 torch extension (inputs device-resident and contiguous, checked with its CHECK_INPUT
 wording) and runs ringattn_fwd of the C ABI on torch's current stream.  Plans (parameters
-+ workspace) are cached inside the extension per parameter set AND stream (at most 16, least
-recently used first out), so forwards on different streams never share a workspace.
++ device tables) are cached inside the extension per parameter set AND stream (at most 16,
+least recently used first out), so forwards on different streams never share a plan.
 """
 import os
 
