@@ -32,7 +32,9 @@
 //           acc-O of :226-232) only when some row's tile max exceeds it by more than
 //           2^kLazyLog2, decided by a wave-uniform branch.  Until then p = exp2((s - m) k2)
 //           may exceed 1 (by at most 2^kLazyLog2, well inside fp16 and bf16 range); O = acc / l
-//           and LSE = (m k2 + log2 l) ln 2 do not depend on the choice of m.
+//           and LSE = (m k2 + log2 l) ln 2 do not depend on the choice of m.  At d = 64, where this
+//           work bounds the kernel, a tile's row maximum is not even computed as long as its
+//           exponentials against the standing reference stay small (softmax_phase).
 //
 //       A tile's work is laid out in time in two phases.  The eight waves sit two per SIMD
 //       (wave w and wave w + 4).  Per tile every wave has an MFMA phase (O^T += V(u)^T P(u)^T, then
@@ -251,14 +253,14 @@ __global__ __launch_bounds__(512, 1) void ring_walk_kernel(const BlockArgs a) {
   };
   // P^T = exp2(S^T k2 - m k2): row sum from the unrounded values (csrc/ring_attention.cu:242),
   // MFMA operands rounded to the storage type (:604)
-  auto exponentials = [&]() {
+  auto exponentials = [&](float (&sums)[4]) {
 #pragma unroll
     for (int t2 = 0; t2 < 2; ++t2) {
       typename E::vec8 pv;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[8 * t2 + e], a.scale_log2, -ms));
-        ls[e & 3] += p;
+        sums[e & 3] += p;
         pv[e] = (typename E::type)p;
       }
       pf[t2] = __builtin_bit_cast(s16x8, pv);
@@ -280,9 +282,32 @@ __global__ __launch_bounds__(512, 1) void ring_walk_kernel(const BlockArgs a) {
     }
   };
   // the softmax phase of the tile whose scores are in sacc
+  // At d = 64 the kernel is bound by this phase (the same VALU work per score as at d = 128 for half the
+  // MFMA work), and the phase runs speculatively: exponentials against the reference as it stands, and the
+  // tile's row maximum is only looked at when some probability came out large (a sum of four of them above
+  // kSpecLimit, which fp16 still holds; an infinity or a NaN also lands here) or a row has no reference yet.
+  // At d = 128 the same change measured 6-9 % slower: the decision then sits at the end of the phase, between
+  // the wave's last VALU result and the first fragment reads of its next MFMA phase.
+  constexpr bool kSpeculate = D == 64;
+  constexpr float kSpecLimit = 16384.f;
   auto softmax_phase = [&]() {
-    move_reference(tile_max());
-    exponentials();
+    if (!kSpeculate) {
+      move_reference(tile_max());
+      exponentials(ls);
+      return;
+    }
+    float sums[4] = {0.f, 0.f, 0.f, 0.f};
+    exponentials(sums);
+    const float largest = fmaxf(fmaxf(sums[0], sums[1]), fmaxf(sums[2], sums[3]));
+    const bool again = !(largest <= kSpecLimit) || m == -INFINITY;
+    if (__builtin_amdgcn_ballot_w64(again) != 0) {
+      move_reference(tile_max());
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sums[i] = 0.f;
+      exponentials(sums);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ls[i] += sums[i];
   };
   auto phase_fence = [&]() { __builtin_amdgcn_sched_barrier(0); };  // keeps the compiler from mixing the phases
   // The MFMA phase of a steady block: O += P(u) V(u), then S(u+1) = K(u+1) Q^T.  Scheduling hint: the

@@ -195,6 +195,11 @@ def test_workload_whole_heads(oracle, name, step_partials):
     Workload("c128", 2, 2, 128, 3, 384, "fp16", 25, True),        # odd rank count
     Workload("p64", 1, 1, 128, 64, 128, "bf16", 26, True),        # maximum number of ranks
     Workload("big_logits", 1, 2, 128, 4, 512, "fp16", 27, False, sigma_qk=3.0),
+    # d = 64 runs its softmax phase speculatively against the reference as it stands: logits whose row maximum
+    # keeps climbing by many powers of two (sigma 9 and 36) make it fall back, also from an overflowed exponential
+    Workload("big_logits_64", 1, 2, 64, 4, 512, "fp16", 28, False, sigma_qk=3.0),
+    Workload("huge_logits_64", 1, 2, 64, 3, 384, "bf16", 29, True, sigma_qk=6.0),
+    Workload("huge_logits_64h", 2, 1, 64, 2, 640, "fp16", 30, False, sigma_qk=6.0),
 ], ids=lambda w: w.name)
 def test_shapes_and_edges_full(oracle, w):
     q, k, v = api.make_qkv_bits(w)

@@ -85,6 +85,8 @@ def test_walk_kernel_runs_two_waves_per_simd_without_spills(tmp_path):
         # partials, three 64-register batches in flight) may around that merge, never in the steady loops
         assert u["ScratchSize [bytes/lane]"] == 0 or not carried, (n, u)
         assert u["VGPRs"] <= 256, (n, u)                       # eight waves per workgroup, one workgroup per compute unit
+        if carried and "Li64E" in n:
+            assert u["VGPRs"] <= 128, (n, u)                   # d = 64: two workgroups per compute unit (+12 % measured)
         # K and V rings; the variants that merge park the partial LSEs of their 256 rows there afterwards
         assert u["LDS Size [bytes/block]"] == (32768 if carried and "Li64E" in n else 65536), (n, u)
         if "Li128E" in n:
