@@ -32,10 +32,10 @@ PEAK_HBM_GBS = 8000.0
 # (bytes, summary under profiles/, kernel_source_id() when it was measured).  The figure is only printed while the
 # kernel source is still the one that was profiled.
 MEASURED_TRAFFIC = {
-    "cfg4": (3486e6, "profiles/ring_walk_kernel_cfg4.md", "6190318dd3a10f05"),
-    "cfg2": (34.2e6, "profiles/ring_walk_kernel_other_workloads.md", "6190318dd3a10f05"),
-    "cfg3": (2189e6, "profiles/ring_walk_kernel_other_workloads.md", "6190318dd3a10f05"),
-    "cfg5": (18260e6, "profiles/ring_walk_kernel_other_workloads.md", "6190318dd3a10f05"),
+    "cfg4": (3499e6, "profiles/ring_walk_kernel_cfg4.md", "494a183db25c449b"),
+    "cfg2": (34.3e6, "profiles/ring_walk_kernel_other_workloads.md", "494a183db25c449b"),
+    "cfg3": (2188e6, "profiles/ring_walk_kernel_other_workloads.md", "494a183db25c449b"),
+    "cfg5": (18260e6, "profiles/ring_walk_kernel_other_workloads.md", "494a183db25c449b"),
 }
 BASELINE_METRIC = "ring-attn fwd TFLOP/s + % bf16 MFMA peak, S=32K d=128 8-step ring, 1 GPU"
 

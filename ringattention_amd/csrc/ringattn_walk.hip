@@ -199,6 +199,16 @@ __global__ __launch_bounds__(512, 1) void ring_walk_kernel(const BlockArgs a) {
     if (decltype(checked)::value && t == kv_tail) load_lds_16(vt, goff_v - surplus(piece_v), vd);
     else load_lds_16(vt, goff_v, vd);
   };
+  // the same for a tile given by address (interior groups keep running pointers instead of recomputing
+  // tile_offset: two scalar instructions per load instead of eighteen)
+  auto issue_k_at = [&](const char* kt, int slot) {
+    const unsigned kd = __builtin_amdgcn_readfirstlane(smem_base + slot * TILE + piece_k * 1024);
+    load_lds_16(kt, goff_k, kd);
+  };
+  auto issue_v_at = [&](const char* vt, int slot) {
+    const unsigned vd = __builtin_amdgcn_readfirstlane(smem_base + (NBUF + slot) * TILE + piece_v * 1024);
+    load_lds_16(vt, goff_v, vd);
+  };
   constexpr std::true_type kChecked{};
   constexpr std::false_type kUnchecked{};
 
@@ -379,15 +389,32 @@ __global__ __launch_bounds__(512, 1) void ring_walk_kernel(const BlockArgs a) {
   auto walk = [&](auto second_c) {
     constexpr bool SECOND = decltype(second_c)::value;
     // STEADY blocks (tiles u+1 and u+2 unmasked or covered by MASKED) have compile-time ring slots
-    auto block = [&](auto slot_c, auto steady, auto masked, int u) {
+    // which tiles this half of the workgroup loads: all waves a piece of each (d = 128), or the first half K and
+    // the second half V (d = 64)
+    constexpr bool LOADS_K = PIECES == WAVES || !SECOND, LOADS_V = PIECES == WAVES || SECOND;
+    const char *k_next = nullptr, *v_next = nullptr;  // interior groups: the next K and the next V tile to load
+    auto block = [&](auto slot_c, auto steady, auto masked, auto interior, int u) {
       constexpr int SLOT = decltype(slot_c)::value;  // u mod 4 (STEADY only)
       constexpr bool STEADY = decltype(steady)::value;
       constexpr bool MASKED = decltype(masked)::value;  // STEADY only: tile u+1 gets the mask
+      constexpr bool INTERIOR = decltype(interior)::value;  // STEADY only: every tile loaded lies inside the chunk
       if (STEADY) {
         // the two tile loads of a block go out next to the softmax phase of the wave (the VALU side has issue
         // slots to spare): K(u+3), K(u+4) in even blocks, V(u+1), V(u+2) in odd ones
         auto issue_loads = [&]() {
-          if ((SLOT & 1) == 0) {
+          if (INTERIOR) {
+            if ((SLOT & 1) == 0) {
+              if (LOADS_K) {
+                issue_k_at(k_next, (SLOT + 3) & 3);
+                issue_k_at(k_next + TILE, SLOT);
+                k_next += 2 * TILE;
+              }
+            } else if (LOADS_V) {
+              issue_v_at(v_next, (SLOT + 1) & 3);
+              issue_v_at(v_next + TILE, (SLOT + 2) & 3);
+              v_next += 2 * TILE;
+            }
+          } else if ((SLOT & 1) == 0) {
             issue_k(u + 3, kUnchecked);
             issue_k(u + 4, kUnchecked);
           } else {
@@ -487,20 +514,34 @@ __global__ __launch_bounds__(512, 1) void ring_walk_kernel(const BlockArgs a) {
       const bool ragged = kv_tail >= 0;
       const int plain_end = ragged ? min(first_masked, kv_tail - 2) : (diag ? first_masked : n_tiles + 1);
       const int masked_end = (diag && !ragged) ? n_tiles + 1 : 0;
+      constexpr std::true_type kYes{};
+      constexpr std::false_type kNo{};
       int u = 0;
+      // interior plain groups: the group at u loads K up to tile u+6 and V up to tile u+5, all inside the chunk
+      k_next = kbase + 3 * TILE;
+      v_next = vbase + 2 * TILE;
+      // (d = 64 only: +9 % on cfg2, whose softmax phase is what a wave spends its issue slots on; at d = 128 the
+      // same change measured 2-6 % slower, as did everything else that shortened the softmax phase there)
+      constexpr bool kInteriorGroups = D == 64;
+      for (; kInteriorGroups && u + 4 < plain_end && u + 6 < n_tiles; u += 4) {
+        block(C0{}, kYes, kNo, kYes, u);
+        block(C1{}, kYes, kNo, kYes, u + 1);
+        block(C2{}, kYes, kNo, kYes, u + 2);
+        block(C3{}, kYes, kNo, kYes, u + 3);
+      }
       for (; u + 4 < plain_end; u += 4) {
-        block(C0{}, std::true_type{}, std::false_type{}, u);
-        block(C1{}, std::true_type{}, std::false_type{}, u + 1);
-        block(C2{}, std::true_type{}, std::false_type{}, u + 2);
-        block(C3{}, std::true_type{}, std::false_type{}, u + 3);
+        block(C0{}, kYes, kNo, kNo, u);
+        block(C1{}, kYes, kNo, kNo, u + 1);
+        block(C2{}, kYes, kNo, kNo, u + 2);
+        block(C3{}, kYes, kNo, kNo, u + 3);
       }
       for (; u + 4 < masked_end; u += 4) {
-        block(C0{}, std::true_type{}, std::true_type{}, u);
-        block(C1{}, std::true_type{}, std::true_type{}, u + 1);
-        block(C2{}, std::true_type{}, std::true_type{}, u + 2);
-        block(C3{}, std::true_type{}, std::true_type{}, u + 3);
+        block(C0{}, kYes, kYes, kNo, u);
+        block(C1{}, kYes, kYes, kNo, u + 1);
+        block(C2{}, kYes, kYes, kNo, u + 2);
+        block(C3{}, kYes, kYes, kNo, u + 3);
       }
-      for (; u < n_tiles; ++u) block(C0{}, std::false_type{}, std::false_type{}, u);
+      for (; u < n_tiles; ++u) block(C0{}, kNo, kNo, kNo, u);
       carried = carry;
       if (keep_state) {
         // the softmax state runs on into the next chunk; with the pipeline carried over as well, the chunk
