@@ -12,7 +12,7 @@ LIB_PATH = os.environ.get("RINGATTN_LIB") or os.path.join(PKG_DIR, "libringattn.
 
 TORCH_LIB_PATH = os.path.join(PKG_DIR, "libringattn_torch.so")
 
-SOURCES = ["ringattn_kernels.hip", "ringattn_walk.hip", "ringattn_api.hip", "ringattn_datagen.cpp"]
+SOURCES = ["ringattn_kernels.hip", "ringattn_walk.hip", "ringattn_walk64.hip", "ringattn_api.hip", "ringattn_datagen.cpp"]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
 HIPCC_FLAGS = [

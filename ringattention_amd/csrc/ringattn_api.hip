@@ -205,7 +205,16 @@ size_t workspace_bytes_of(const ringattn_params* p, const Derived& d) {
 struct TableSlice {
   int seg_begin = 0, seg_count = 0;
   int q_tiles_max = 0;  // kWalkM-row tiles of the longest segment
+  bool wide = false;    // every KV range of the slice suits ring_walk64_kernel
 };
+
+// ring_walk64_kernel walks whole 32-key tiles and steps its load streams four tiles at a time: a KV range must
+// be a multiple of 32 keys and hold at least 128.
+static bool walk64_takes(const ringattn::SegItem& it) { return it.kv_len % 32 == 0 && it.kv_len >= 128; }
+static bool walk64_enabled() {
+  const char* e = std::getenv("RINGATTN_WIDE");
+  return e && e[0] == '1';
+}
 
 struct ringattn_plan {
   ringattn_params p{};
@@ -329,6 +338,8 @@ void build_schedule(ringattn_plan* pl) {
     }
   }
   pl->fwd_items = (int)pl->h_items.size();
+  pl->fwd.wide = true;
+  for (const auto& it : pl->h_segitems) pl->fwd.wide = pl->fwd.wide && walk64_takes(it);
   // Workgroup order of the forward.  Heads are dealt to the 8 XCDs round-robin; an XCD runs
   // the segments of one head after the other (busiest first within a head), so the ranks of
   // a head, which read the same K and V, follow each other through that XCD's L2.  Only when
@@ -430,7 +441,10 @@ int launch_slice(const ringattn_plan* pl, const TableSlice& sl, ringattn::BlockA
   a.items = pl->d_segitems;
   a.n_segs = sl.seg_count;
   a.q_tiles_max = sl.q_tiles_max;
-  RA_HIP(ringattn::launch_walk(a, pl->p.dtype, pl->p.dim, stream));
+  if (sl.wide && pl->p.dim == 128 && pl->d.S >= 512 && a.mode == ringattn::kBlockCarryState && walk64_enabled())
+    RA_HIP(ringattn::launch_walk64(a, pl->p.dtype, stream));
+  else
+    RA_HIP(ringattn::launch_walk(a, pl->p.dtype, pl->p.dim, stream));
   return RINGATTN_OK;
 }
 
@@ -562,7 +576,10 @@ int run_rank_call(const RankCall& rc, void* scratch, const void* q, const void* 
   a.q_tiles_max = q_tiles_of(c);
   a.bh_stride = (int64_t)c * dim;  // q and out hold this rank's rows only; k and v the whole sequence
   a.S = c;
-  RA_HIP(ringattn::launch_walk(a, rc.p.dtype, dim, stream));
+  bool wide = dim == 128 && rc.d.S >= 512 && walk64_enabled();
+  for (int i = 0; i < n_parts; ++i) wide = wide && walk64_takes(rc.pack.items[i]);
+  if (wide) RA_HIP(ringattn::launch_walk64(a, rc.p.dtype, stream));
+  else RA_HIP(ringattn::launch_walk(a, rc.p.dtype, dim, stream));
   return RINGATTN_OK;
 }
 
