@@ -19,13 +19,12 @@ Register map (fixed; the C++ side hands its values over in exactly these registe
     v[64:95]    probabilities (B operands), two buffers: buffer f, block b, half t2 at v[64 + 16 f + 8 b + 4 t2 .. +3]
     v[96:127]   the eight K fragments of a tile; v[128:159] the eight V^T fragments
     v[160:175]  LDS offsets of the K fragments (8), of the V^T fragments (4), global offsets of this wave's tile pieces (K 2, V 2)
-    v[176:189]  m (2), m k2 (2), row sums (2 x 4), cand (2);  v[192:199] temporaries
+    v[176:187]  m (2), m k2 (2), row sums (2 x 4);  v[192:199] temporaries
     v[200:231]  the exponentials of the tile before rounding, v[232:239] their sums (four per block)
     s[36:37] K load pointer, s38 tiles left in its chunk, s39 LDS address of the list entry of the chunk after it;
     s[40:43] the same for V;  s[44:45] / s[46:47] first row of the head in K / V, s48 k2, s49 / s50 LDS address of this
     wave's first piece in K / V ring slot 0, s51 the iteration u, s52 the first u whose score tile u+1 is not computed,
-    s53 why the loop was left (2: the workgroup's last iteration is done; 3, 4: the exponentials of tile u have to be
-    redone against a new reference), s54 the first u whose score tile gets the causal mask, s55 the last iteration;
+    s53 set to 2 when the workgroup's last iteration is done, s54 the first u whose score tile gets the causal mask, s55 the last iteration;
     v[190:191] mask limits of the two blocks
 """
 import os
@@ -96,8 +95,9 @@ CAND = lambda b: "v%d" % (188 + b)
 TMP = lambda i: "v%d" % (192 + i)
 PX = lambda b, e: "v%d" % (200 + 16 * b + e)      # exponentials of the tile, unrounded
 TS = lambda b, i: "v%d" % (232 + 4 * b + i)       # their sums, four per block
-SPEC = _knob('SPEC', 1)   # 1: no row maximum in the loop; the exponentials are taken against the reference as it
-                          # stands and the loop is left (the tile redone) when a sum of four of them exceeds 2^14
+# There is no row maximum in the loop: the exponentials are taken against the reference as it stands, and only when a
+# sum of four of them exceeds 2^14 (or is not a number) is the row maximum looked at, the reference moved and the
+# tile's exponentials redone (redo_routine)
 
 S_KHEAD, S_VHEAD = (44, 45), (46, 47)
 S_K2, S_LDSK, S_LDSV = "s48", "s49", "s50"
@@ -171,6 +171,86 @@ def k_prereads(i_next):
     return ["ds_read_b128 %s, %s offset:%d" % (KF(ks), KOFF(ks), slot * TILE) for ks in range(PREREAD)]
 
 
+def exp_stream(cur, cvt):
+    """P = exp2(S k2 - m k2) of the score buffer `cur`, both blocks interleaved element by element: the unrounded
+    values to PX, their sums (four per block) to TS, the rounded pairs to the probability buffer `cur`.  The three
+    steps of an element (scale-and-subtract, exponential, sum / conversion) are DEPTH elements apart."""
+    elems = [(b, e) for e in range(16) for b in range(2)]
+    valu = []
+    DEPTH = _knob('DEPTH', 8)
+
+    def emit_step(kind, k):
+        b, e = elems[k]
+        if kind == 0:
+            valu.append("v_fma_f32 %s, %s, %s, -%s" % (PX(b, e), Sreg(cur, b, e), S_K2, MS(b)))
+        elif kind == 1:
+            valu.append("v_exp_f32 %s, %s" % (PX(b, e), PX(b, e)))
+        else:
+            if e >= 4:
+                first = PX(b, e - 4) if e < 8 else TS(b, e & 3)
+                valu.append("v_add_f32 %s, %s, %s" % (TS(b, e & 3), first, PX(b, e)))
+            if e & 1:   # the pair (e - 1, e) is complete
+                valu.append("%s %s, %s, %s" % (cvt, Preg(cur, b, e // 8, (e % 8) // 2), PX(b, e - 1), PX(b, e)))
+    for k in range(len(elems) + 2 * DEPTH):
+        if k < len(elems):
+            emit_step(0, k)
+        if 0 <= k - DEPTH < len(elems):
+            emit_step(1, k - DEPTH)
+        if 0 <= k - 2 * DEPTH < len(elems):
+            emit_step(2, k - 2 * DEPTH)
+    return valu
+
+
+def redo_routine(cur, cvt):
+    """Out of line: the exponentials of the tile in score buffer `cur` came out too large for the standing reference
+    (a sum of four above 2^14).  All MFMAs of the iteration are issued and acc-O holds the tiles before this one, so
+    the reference moves to the row maximum at once -- l and acc-O rescaled as in csrc/ring_attention.cu:226-232 -- and
+    the exponentials are taken again.  s57 says where to go back to."""
+    out = ["85%d:" % cur, "s_nop 15"]
+    for stp in range(4):
+        for b in range(2):
+            for c in range(2):
+                t = TMP(2 * b + c)
+                first = M(b) if stp == 0 else t
+                out.append("v_max3_f32 %s, %s, %s, %s" % (t, first, Sreg(cur, b, 4 * stp + 2 * c), Sreg(cur, b, 4 * stp + 2 * c + 1)))
+    for b in range(2):
+        out.append("v_max_f32 %s, %s, %s" % (TMP(2 * b), TMP(2 * b), TMP(2 * b + 1)))
+    for b in range(2):
+        out.append("v_mov_b32 %s, %s" % (TMP(2 * b + 1), TMP(2 * b)))
+    for b in range(2):
+        out += ["s_nop 1", "v_permlane32_swap_b32 %s, %s" % (TMP(2 * b), TMP(2 * b + 1))]
+    out.append("s_nop 1")
+    for b in range(2):
+        out.append("v_max_f32 %s, %s, %s" % (M(b), TMP(2 * b), TMP(2 * b + 1)))        # the new reference
+    for b in range(2):
+        out.append("v_mul_f32 %s, %s, %s" % (TMP(4 + b), S_K2, M(b)))                  # m k2
+    for b in range(2):
+        out.append("v_sub_f32 %s, %s, %s" % (TMP(6 + b), MS(b), TMP(4 + b)))           # old m k2 - new m k2
+    for b in range(2):
+        out.append("v_exp_f32 %s, %s" % (TMP(6 + b), TMP(6 + b)))                      # alpha
+    for b in range(2):
+        out.append("v_mov_b32 %s, %s" % (MS(b), TMP(4 + b)))
+    out.append("s_nop 1")
+    for b in range(2):
+        for q in range(4):
+            out.append("v_mul_f32 %s, %s, %s" % (LS(b, q), LS(b, q), TMP(6 + b)))
+    # acc-O, eight registers at a time through the (dead) exponential buffer
+    for b in range(2):
+        for r0 in range(0, 64, 8):
+            for r in range(8):
+                out.append("v_accvgpr_read_b32 %s, a%d" % (PX(0, r), 64 * b + r0 + r))
+            for r in range(8):
+                out.append("v_mul_f32 %s, %s, %s" % (PX(0, r), PX(0, r), TMP(6 + b)))
+            for r in range(8):
+                out.append("v_accvgpr_write_b32 a%d, %s" % (64 * b + r0 + r, PX(0, r)))
+    out += exp_stream(cur, cvt)
+    for site, c in _redo:
+        if c == cur:
+            out += ["s_cmp_eq_u32 %s, %d" % (S_T(1), site), "s_cbranch_scc1 86%02db" % site]
+    out.append("s_branch 199f")   # not reached
+    return out
+
+
 def iteration(i, mfma, cvt, do_qk=True, do_sm=True, do_pv=True):
     """Iteration u = 8 g + i of the steady loop: S(u+1) = K(u+1) Q^T, P(u) from S(u), O += P(u-1) V(u-1).
     Without do_qk / do_sm: the iterations after a wave's last score tile (no instruction order to speak of)."""
@@ -205,36 +285,9 @@ def iteration(i, mfma, cvt, do_qk=True, do_sm=True, do_pv=True):
                 mf.append(("%s %s, %s, %s, %s" % (mfma, O(b, db), VF(idx), Pvec(nxt, b, t2), O(b, db)), len(reads) - 1))
     need_at = [min(j for j, (_, r) in enumerate(mf) if r >= k) for k in range(len(reads))]
 
-    # exponentials of S(u) (buffer cur), both blocks interleaved element by element; F -> X -> A three apart
-    elems = [(b, e) for e in range(16) for b in range(2)] if do_sm else []
-    valu = []
-    DEPTH = _knob('DEPTH', 8)   # instructions of other elements between the three steps of one element
-    def emit_step(kind, k):
-        b, e = elems[k]
-        src = Sreg(cur, b, e)
-        dst = PX(b, e) if SPEC else src     # speculative: the scores stay intact, the tile may have to be redone
-        if kind == 0:
-            valu.append("v_fma_f32 %s, %s, %s, -%s" % (dst, src, S_K2, MS(b)))
-        elif kind == 1:
-            valu.append("v_exp_f32 %s, %s" % (dst, dst))
-        else:
-            if not SPEC:
-                valu.append("v_add_f32 %s, %s, %s" % (LS(b, e & 3), LS(b, e & 3), dst))
-            elif e >= 4:
-                first = PX(b, e - 4) if e < 8 else TS(b, e & 3)
-                valu.append("v_add_f32 %s, %s, %s" % (TS(b, e & 3), first, dst))
-            if e & 1:   # the pair (e - 1, e) is complete
-                lo = PX(b, e - 1) if SPEC else Sreg(cur, b, e - 1)
-                valu.append("%s %s, %s, %s" % (cvt, Preg(cur, b, e // 8, (e % 8) // 2), lo, dst))
-    for k in range(len(elems) + 2 * DEPTH if elems else 0):
-        if k < len(elems):
-            emit_step(0, k)
-        if 0 <= k - DEPTH < len(elems):
-            emit_step(1, k - DEPTH)
-        if 0 <= k - 2 * DEPTH < len(elems):
-            emit_step(2, k - 2 * DEPTH)
+    valu = exp_stream(cur, cvt) if do_sm else []
     spec_check = []
-    if SPEC and do_sm:
+    if do_sm:
         for b in range(2):
             spec_check.append("v_max3_f32 %s, %s, %s, %s" % (TMP(b), TS(b, 0), TS(b, 1), TS(b, 2)))
         for b in range(2):
@@ -247,34 +300,7 @@ def iteration(i, mfma, cvt, do_qk=True, do_sm=True, do_pv=True):
                 spec_check.append("v_add_f32 %s, %s, %s" % (LS(b, q), LS(b, q), TS(b, q)))
     n_exp_valu = len(valu)
     tail = []
-    if do_qk and not _knob('NOMAX', 0) and not SPEC:
-        # the mask limits move on by a tile
-        for b in range(2):
-            valu.append("v_subrev_u32_e32 %s, 32, %s" % (VLIM(b), VLIM(b)))
-        # row maximum of S(u+1) (buffer nxt): per block two chains of v_max3, one exchange between the halves of the wave
-        for stp in range(4):
-            for b in range(2):
-                for c in range(2):
-                    t = TMP(2 * b + c)
-                    first = M(b) if stp == 0 else t
-                    valu.append("v_max3_f32 %s, %s, %s, %s" % (t, first, Sreg(nxt, b, 4 * stp + 2 * c), Sreg(nxt, b, 4 * stp + 2 * c + 1)))
-        for b in range(2):
-            valu.append("v_max_f32 %s, %s, %s" % (TMP(2 * b), TMP(2 * b), TMP(2 * b + 1)))
-        for b in range(2):
-            valu.append("v_mov_b32 %s, %s" % (TMP(2 * b + 1), TMP(2 * b)))
-        for b in range(2):
-            tail += ["s_nop 1", "v_permlane32_swap_b32 %s, %s" % (TMP(2 * b), TMP(2 * b + 1))]
-        tail += ["s_nop 1"]
-        for b in range(2):
-            tail.append("v_max_f32 %s, %s, %s" % (CAND(b), TMP(2 * b), TMP(2 * b + 1)))
-        # a reference moves when cand k2 - m k2 > 8 for some row: leave the loop (the C++ side moves it)
-        for b in range(2):
-            tail.append("v_fma_f32 %s, %s, %s, -%s" % (TMP(4 + b), CAND(b), S_K2, MS(b)))
-        tail.append("v_max_f32 %s, %s, %s" % (TMP(4), TMP(4), TMP(5)))
-        tail.append("v_cmp_lt_f32_e32 vcc, 0x41000000, %s" % TMP(4))
-    if do_qk and _knob('NOMAX', 0):
-        tail.append("v_cmp_lt_f32_e32 vcc, 0x7f800000, %s" % M(0))   # never
-    if do_qk and SPEC:
+    if do_qk:   # the mask limits move on by a tile
         for b in range(2):
             valu.append("v_subrev_u32_e32 %s, 32, %s" % (VLIM(b), VLIM(b)))
 
@@ -320,7 +346,7 @@ def iteration(i, mfma, cvt, do_qk=True, do_sm=True, do_pv=True):
         if ln == "SPECBRANCH":
             site = len(_redo)
             _redo.append((site, cur))
-            out.append("s_cbranch_vccnz 8%02df" % site)
+            out += ["s_cbranch_vccnz 8%02df" % site, "86%02d:" % site]
         else:
             out.append(ln)
     out += tail
@@ -368,11 +394,10 @@ def loop_text(mfma, cvt):
     for i in range(UNROLL):
         lines += mask_code(i)
     lines += chunk_changes()
-    # the exponentials of tile u came out too large for the standing reference: out, with iteration u complete but
-    # for them (all its MFMAs are issued); 3: the scores of tile u are in buffer 0 and those of tile u+1 in buffer 1,
-    # 4: the other way round
     for site, cur in _redo:
-        lines += ["8%02d:" % site, "s_nop 15", "s_mov_b32 %s, %d" % (S_FAR, 3 + cur), "s_branch 199f"]
+        lines += ["8%02d:" % site, "s_mov_b32 %s, %d" % (S_T(1), site), "s_branch 85%df" % cur]
+    for cur in range(2):
+        lines += redo_routine(cur, cvt)
     lines.append("198:")
     lines.append("s_mov_b32 %s, 2" % S_FAR)
     lines.append("199:")
@@ -388,15 +413,15 @@ def operands():
     for b in range(2):
         outs.append('"+{%s}"(sacc[%d])' % (Svec(0, b), b))
     for b in range(2):
-        outs.append('"+{%s}"(sx[%d])' % (Svec(1, b), b))
-    for b in range(2):
         for t2 in range(2):
             outs.append('"+{%s}"(pprev[%d][%d])' % (Pvec(1, b, t2), b, t2))
     for b in range(2):
         for i in range(4):
             outs.append('"+{%s}"(ls[%d][%d])' % (LS(b, i), b, i))
     for b in range(2):
-        outs.append('"+{%s}"(cand[%d])' % (CAND(b), b))
+        outs.append('"+{%s}"(m[%d])' % (M(b), b))
+    for b in range(2):
+        outs.append('"+{%s}"(ms[%d])' % (MS(b), b))
     for st, n in ((KST, "k"), (VST, "v")):
         outs += ['"+{%s}"(%s_lo)' % (st.lo, n), '"+{%s}"(%s_hi)' % (st.hi, n), '"+{%s}"(%s_left)' % (st.left, n),
                  '"+{%s}"(%s_next)' % (st.next, n)]
@@ -414,14 +439,10 @@ def operands():
         ins.append('"{%s}"(goff_k[%d])' % (GOFFK(j), j))
     for j in range(2):
         ins.append('"{%s}"(goff_v[%d])' % (GOFFV(j), j))
-    for b in range(2):
-        ins.append('"{%s}"(m[%d])' % (M(b), b))
-    for b in range(2):
-        ins.append('"{%s}"(ms[%d])' % (MS(b), b))
     ins += ['"{%s}"(kh_lo)' % KST.head[0], '"{%s}"(kh_hi)' % KST.head[1], '"{%s}"(vh_lo)' % VST.head[0], '"{%s}"(vh_hi)' % VST.head[1],
             '"{%s}"(k2_bits)' % S_K2, '"{%s}"(lds_dst_k)' % S_LDSK, '"{%s}"(lds_dst_v)' % S_LDSV,
             '"{%s}"(asm_stop)' % S_STOP, '"{%s}"(asm_mw1)' % S_MW1, '"{%s}"(asm_n)' % S_N]
-    clob = ["v%d" % r for r in list(range(64, 80)) + list(range(96, 160)) + list(range(192, 240))]
+    clob = ["v%d" % r for r in list(range(32, 80)) + list(range(96, 160)) + [188, 189] + list(range(192, 240))]
     clob += ["s56", "s57", "vcc", "scc", "m0", "memory"]
     return outs, ins, clob
 

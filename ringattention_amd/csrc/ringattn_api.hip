@@ -211,9 +211,10 @@ struct TableSlice {
 // ring_walk64_kernel walks whole 32-key tiles and steps its load streams four tiles at a time: a KV range must
 // be a multiple of 32 keys and hold at least 128.
 static bool walk64_takes(const ringattn::SegItem& it) { return it.kv_len % 32 == 0 && it.kv_len >= 128; }
+// RINGATTN_WIDE=0 in the environment keeps every forward on ring_walk_kernel (for comparisons)
 static bool walk64_enabled() {
   const char* e = std::getenv("RINGATTN_WIDE");
-  return e && e[0] == '1';
+  return !(e && e[0] == '0');
 }
 
 struct ringattn_plan {

@@ -373,74 +373,25 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
   const unsigned vh_lo = uni((unsigned)(uintptr_t)v_head), vh_hi = uni((unsigned)((uintptr_t)v_head >> 32));
   const unsigned k2_bits = uni(__builtin_bit_cast(unsigned, a.scale_log2));
 
-  int u = 0;
-  while (u <= N) {
-    // The hand-scheduled loop (ringattn_walk64_loop.inc) takes over at a multiple of eight (its ring slots are
-    // immediates) and runs to the workgroup's last iteration: every iteration whose score tile u+1 this wave
-    // computes -- masking the tiles of the diagonal chunk that need it --, the wave's last two iterations, and then
-    // only the wave's share of the loads and the barriers.  It comes back early when the exponentials of a tile have
-    // to be redone against a new reference.
-    if ((u & 7) == 0 && !pend && u + 1 < Ew) {
-      unsigned asm_u = uni((unsigned)u), asm_far = 0;
-      const unsigned asm_stop = uni((unsigned)(Ew - 1)), asm_mw1 = uni((unsigned)(Mw - 1));
-      f32x16 sx[2];  // the loop's second score buffer
+  // The hand-scheduled loop (ringattn_walk64_loop.inc) runs all iterations of the workgroup, 0 to N: every iteration
+  // whose score tile u+1 this wave computes -- masking the tiles of the diagonal chunk that need it --, the wave's last
+  // two iterations, and then only the wave's share of the loads and the barriers.  A wave with no second score tile
+  // walks the iterations in plain code.
+  if (1 < Ew) {
+    const int u = 0;  // where the loop starts
+    unsigned asm_u = 0, asm_far = 0;
+    const unsigned asm_stop = uni((unsigned)(Ew - 1)), asm_mw1 = uni((unsigned)(Mw - 1));
+    int vlim[2];
 #pragma unroll
-      for (int b = 0; b < 2; ++b) sx[b] = sacc[b];
-      int vlim[2];
-#pragma unroll
-      for (int b = 0; b < 2; ++b) vlim[b] = diag_rows + 64 * wave + 32 * b + n - 4 * h - (u + 1 - diag_base) * BN;
-      const uint64_t kp = (uint64_t)(uintptr_t)k_head + kst.off, vp = (uint64_t)(uintptr_t)v_head + vst.off;
-      unsigned k_lo = uni((unsigned)kp), k_hi = uni((unsigned)(kp >> 32)), v_lo = uni((unsigned)vp), v_hi = uni((unsigned)(vp >> 32));
-      unsigned k_left = uni((unsigned)kst.left), v_left = uni((unsigned)vst.left);
-      unsigned k_next = uni(smem_base + kListAt + 8 * (kst.idx + 1)), v_next = uni(smem_base + kListAt + 8 * (vst.idx + 1));
-      const unsigned asm_n = uni((unsigned)N);
+    for (int b = 0; b < 2; ++b) vlim[b] = diag_rows + 64 * wave + 32 * b + n - 4 * h - (u + 1 - diag_base) * BN;
+    const uint64_t kp = (uint64_t)(uintptr_t)k_head + kst.off, vp = (uint64_t)(uintptr_t)v_head + vst.off;
+    unsigned k_lo = uni((unsigned)kp), k_hi = uni((unsigned)(kp >> 32)), v_lo = uni((unsigned)vp), v_hi = uni((unsigned)(vp >> 32));
+    unsigned k_left = uni((unsigned)kst.left), v_left = uni((unsigned)vst.left);
+    unsigned k_next = uni(smem_base + kListAt + 8 * (kst.idx + 1)), v_next = uni(smem_base + kListAt + 8 * (vst.idx + 1));
+    const unsigned asm_n = uni((unsigned)N);
 #include "ringattn_walk64_loop.inc"
-      kst.off = k_lo - kh_lo;
-      vst.off = v_lo - vh_lo;
-      kst.left = (int)k_left;
-      vst.left = (int)v_left;
-      kst.idx = (int)(k_next - (smem_base + kListAt)) / 8 - 1;
-      vst.idx = (int)(v_next - (smem_base + kListAt)) / 8 - 1;
-      u = (int)asm_u;
-      if (asm_far >= 3) {
-        // The loop takes the exponentials against the reference as it stands and has found those of tile u too
-        // large for it (a sum of four above 2^14).  Iteration u is complete but for them: acc-O holds the tiles up to
-        // u-1, so the reference moves at once (csrc/ring_attention.cu:226-232), and the exponentials are redone.
-        if (asm_far == 4) {
-#pragma unroll
-          for (int b = 0; b < 2; ++b) {
-            const f32x16 t = sacc[b];
-            sacc[b] = sx[b];
-            sx[b] = t;
-          }
-        }
-#pragma unroll
-        for (int b = 0; b < 2; ++b) {
-          cand[b] = tile_max(sacc[b], m[b]);
-          const float cs = (cand[b] == -INFINITY) ? 0.f : cand[b] * a.scale_log2;
-          const float alpha = __builtin_amdgcn_exp2f(m[b] * a.scale_log2 - cs);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) ls[b][i] *= alpha;
-#pragma unroll
-          for (int db = 0; db < DB; ++db) oacc[b][db] *= alpha;
-          m[b] = cand[b];
-          ms[b] = cs;
-        }
-        exps(sacc, pprev);
-#pragma unroll
-        for (int b = 0; b < 2; ++b) sacc[b] = sx[b];
-        ++u;
-      }
-      if (asm_far != 2 && u < Ew) {
-        // the scores the loop hands back have not been looked at: the usual check of the reference
-        cand[0] = tile_max(sacc[0], m[0]);
-        cand[1] = tile_max(sacc[1], m[1]);
-        if (far_now()) settle(true);
-      }
-    } else {
-      general(u);
-      ++u;
-    }
+  } else {
+    for (int u = 0; u <= N; ++u) general(u);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   if (pend) settle(false);
