@@ -38,7 +38,7 @@ TILE = 8192
 NBUF = 8
 ROWB = 256
 UNROLL = 8      # iterations per trip: ring slots are immediates
-LEAD = _knob('LEAD', 6)        # a fragment read is issued this many MFMAs ahead of the MFMA that needs it
+LEAD = _knob('LEAD', 3)        # a fragment read is issued this many MFMAs ahead of the MFMA that needs it
 HEAD_VALU = _knob('HEAD', 4)   # vector instructions in front of the first MFMA of an iteration
 PREREAD = _knob('PREREAD', 4)     # K fragments of the next iteration read at the end of this one
 
@@ -131,13 +131,14 @@ def tile_load(st, slot, goff):
     """Both pieces of one tile, then the step of the stream to the next tile (the change of chunk is out of line)."""
     site = len(_sites)
     _sites.append((site, st))
+    ld = "s_nop 0 ;" if _knob('NOLOADS', 0) else ""   # timing only
     return [
         "s_add_u32 m0, %s, %d" % (st.lds, slot * TILE),
         "s_sub_u32 %s, %s, 1" % (st.left, st.left),
-        "global_load_lds_dwordx4 %s, %s" % (goff(0), st.ptr),
+        ld + "global_load_lds_dwordx4 %s, %s" % (goff(0), st.ptr),
         "s_add_u32 m0, %s, %d" % (st.lds, slot * TILE + 1024),
         "s_nop 0",
-        "global_load_lds_dwordx4 %s, %s" % (goff(1), st.ptr),
+        ld + "global_load_lds_dwordx4 %s, %s" % (goff(1), st.ptr),
         "s_add_u32 %s, %s, %d" % (st.lo, st.lo, TILE),
         "s_addc_u32 %s, %s, 0" % (st.hi, st.hi),
         "s_cmp_eq_u32 %s, 0" % st.left,
@@ -257,14 +258,21 @@ def iteration(i, mfma, cvt, do_qk=True, do_sm=True, do_pv=True):
     cur, nxt = i & 1, (i & 1) ^ 1
     kslot, vslot = (i + 1) % NBUF, (i + NBUF - 1) % NBUF
     out = []
+    # the barrier of the pair of iterations and this iteration's tile loads: in front of everything, or (MISC_AT > 0,
+    # full iterations only) worked in behind the first MFMAs.  The K fragments the first MFMAs use were landed a
+    # barrier ago; the V fragments of this iteration are only read behind this barrier.
+    misc = []
     if i % 2 == 0:
-        out += ["s_waitcnt vmcnt(12)"] + ([] if _knob('NOBARRIER', 0) else ["s_barrier"])
-        out += tile_load(KST, (i + 7) % NBUF, GOFFK)
-        out += tile_load(KST, i % NBUF, GOFFK)
+        misc += ["s_waitcnt vmcnt(12)"] + ([] if _knob('NOBARRIER', 0) else ["s_barrier"])
+        misc += tile_load(KST, (i + 7) % NBUF, GOFFK)
+        misc += tile_load(KST, i % NBUF, GOFFK)
     else:
-        out += tile_load(VST, (i + 4) % NBUF, GOFFV)
-        out += tile_load(VST, (i + 5) % NBUF, GOFFV)
-
+        misc += tile_load(VST, (i + 4) % NBUF, GOFFV)
+        misc += tile_load(VST, (i + 5) % NBUF, GOFFV)
+    MISC_AT = _knob('MISC_AT', 2) if (do_qk and do_pv) else 0
+    if not MISC_AT:
+        out += misc
+        misc = []
     # ---- the three instruction streams of the iteration
     mf = []   # (text, index of the last fragment read it needs)
     reads = []  # fragment reads in the order they are issued
@@ -285,7 +293,7 @@ def iteration(i, mfma, cvt, do_qk=True, do_sm=True, do_pv=True):
                 mf.append(("%s %s, %s, %s, %s" % (mfma, O(b, db), VF(idx), Pvec(nxt, b, t2), O(b, db)), len(reads) - 1))
     need_at = [min(j for j, (_, r) in enumerate(mf) if r >= k) for k in range(len(reads))]
 
-    valu = exp_stream(cur, cvt) if do_sm else []
+    valu = exp_stream(cur, cvt) if (do_sm and not _knob('NOEXP', 0)) else []
     spec_check = []
     if do_sm:
         for b in range(2):
@@ -317,28 +325,54 @@ def iteration(i, mfma, cvt, do_qk=True, do_sm=True, do_pv=True):
             issued += 1
         return res
 
+    if _knob('NOREADS', 0):
+        import re as _re   # timing only: the products run on zero fragments
+        reads = ["v_mov_b32 v%s, 0" % _re.search(r"v\[(\d+):", r).group(1) for r in reads]
     out += issue_reads_upto(0)
     vi = 0
     out += valu[vi:vi + HEAD_VALU]
     vi += HEAD_VALU
     masked = False
     waited = -1   # fragment reads up to this index are known to have returned
+    BUDGET = _knob('BUDGET', 0)   # > 0: cycles of other work behind an MFMA (v_exp 8, anything else 4); 0: by count
     for j, (text, r) in enumerate(mf):
+        spent = 0
         if r > waited or _knob('WAITALL', 0):
             out.append("s_waitcnt lgkmcnt(%d)" % min(issued - (r + 1), 15))
             waited = r
+            spent += 4
         out.append(text)
-        out += issue_reads_upto(j + 1)
+        more = issue_reads_upto(j + 1)
+        out += more
+        spent += 4 * len(more)
         if do_qk and j == MASK_AT:
             # tile u+1 lies in this wave's masked range: the mask is applied out of line
             out += ["s_cmp_ge_i32 %s, %s" % (S_C, S_MW1), "s_cbranch_scc1 5%d0f" % i, "6%d0:" % i]
             masked = True
-        share = 4 if j % 2 == 0 else 5
-        for _ in range(share):
-            # the row-maximum instructions only once the mask has had its chance
-            if vi < len(valu) and (vi < n_exp_valu or masked or not do_qk):
-                out.append(valu[vi])
-                vi += 1
+            spent += 8
+        share = _knob('SHARE_A', 3) if j % 2 == 0 else _knob('SHARE_B', 4)
+        n_here = 0
+        if MISC_AT and j + 1 >= MISC_AT:
+            take = _knob('MISC_N', 3)
+            while misc and take > 0:
+                ln = misc.pop(0)
+                out.append(ln)
+                if not ln.endswith(":"):
+                    take -= 1
+                    n_here += 1
+            # a label must not be separated from the branch in front of it by later insertions: flush a dangling one
+            while misc and misc[0].endswith(":"):
+                out.append(misc.pop(0))
+        while vi < len(valu) and (vi < n_exp_valu or masked or not do_qk):
+            # (the mask limits only move on once the mask has had its chance)
+            cost = 8 if valu[vi].startswith("v_exp") else 4
+            if (BUDGET and spent + cost > BUDGET) or (not BUDGET and n_here >= share):
+                break
+            out.append(valu[vi])
+            vi += 1
+            n_here += 1
+            spent += cost
+    assert not misc, "the tile loads did not fit behind the MFMAs"
     out += valu[vi:]
     if do_qk:
         out += k_prereads((i + 1) % UNROLL)
@@ -350,6 +384,8 @@ def iteration(i, mfma, cvt, do_qk=True, do_sm=True, do_pv=True):
         else:
             out.append(ln)
     out += tail
+    if _knob('SLEEP', 0):
+        out.append("s_sleep %d" % _knob('SLEEP', 0))   # experiment: idle cycles (64 each)
     out.append("s_add_u32 %s, %s, 1" % (S_C, S_C))
     return out
 
