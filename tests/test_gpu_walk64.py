@@ -1,0 +1,104 @@
+"""ring_walk64_kernel (64 query rows per wave, d = 128, carried softmax state; ringattn_walk64.hip) against the CPU
+oracle on inputs chosen for its own corner cases, and against ring_walk_kernel on the same inputs.
+
+The kernel takes the exponentials of a tile against the reference maximum as it stands and only looks at the row
+maximum (moving the reference, rescaling l and acc-O as in csrc/ring_attention.cu:226-232, redoing the tile) when a sum
+of four of them exceeds 2^14.  Logits that keep rising along the key sequence force that path again and again: in the
+steady iterations, in the masked tiles of a diagonal chunk and in a wave's last iterations.  Same tolerances as
+everywhere: max-abs 1e-2 on O, 1e-3 relative on LSE (test_gpu_parity.check_rows)."""
+import numpy as np
+import pytest
+import torch
+
+from np_reference import bits_to_float64, float32_to_bits
+from ringattention_amd import api
+from ringattention_amd.configs import Workload
+from test_gpu_parity import check_rows, forward
+
+pytestmark = pytest.mark.gpu
+
+
+def rising_logits(w, slope, period=0):
+    """Q, K, V of workload `w` with one coordinate of K growing along the sequence (or sawtooth-wise with `period`)
+    and the same coordinate of Q fixed at 4: logit(q, key j) grows by 4 * slope * scale per key."""
+    q, k, v = api.make_qkv_bits(w)
+    qf = bits_to_float64(q, w.dtype).astype(np.float32)
+    kf = bits_to_float64(k, w.dtype).astype(np.float32)
+    j = np.arange(w.seq, dtype=np.float32)
+    if period:
+        j = j % period
+    qf[..., 0] = 4.0
+    kf[..., 0] = slope * j
+    return float32_to_bits(qf, w.dtype).reshape(q.shape), float32_to_bits(kf, w.dtype).reshape(k.shape), v
+
+
+@pytest.mark.parametrize("w,slope,period", [
+    # the row maximum climbs by about 400 (natural units) over the sequence: dozens of reference moves per row
+    (Workload("rise_nc", 1, 2, 128, 4, 1024, "bf16", 41, False), 0.28, 0),
+    (Workload("rise_c", 1, 2, 128, 4, 1024, "bf16", 42, True), 0.28, 0),
+    (Workload("rise_c16", 2, 1, 128, 2, 1280, "fp16", 43, True), 0.1, 0),
+    # a sawtooth: the maximum jumps at every tooth's end and nothing later in the tooth reaches it
+    (Workload("saw_nc", 1, 3, 128, 3, 768, "fp16", 44, False), 0.4, 300),
+    # steep enough for the exponentials to overflow to infinity against a stale reference
+    (Workload("steep_c", 1, 1, 128, 2, 1024, "bf16", 45, True), 4.0, 0),
+], ids=lambda x: x.name if isinstance(x, Workload) else None)
+def test_reference_moves_inside_the_hand_scheduled_loop(oracle, w, slope, period):
+    q, k, v = rising_logits(w, slope, period)
+    out, lse = forward(w, q, k, v)
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    check_rows(oracle, w, q, k, v, out, lse, np.arange(w.rows))
+
+
+@pytest.mark.parametrize("w", [
+    Workload("w_nc", 2, 3, 128, 4, 512, "bf16", 51, False),
+    Workload("w_c", 1, 4, 128, 8, 256, "fp16", 52, True),          # 8-tile chunks: a change of chunk every other trip
+    Workload("w_c1", 1, 2, 128, 1, 2048, "bf16", 53, True),        # one chunk, all of it diagonal
+    Workload("w_min", 1, 2, 128, 4, 128, "bf16", 54, True),        # the shortest chunks the kernel takes (4 tiles)
+    Workload("w_big", 1, 2, 128, 2, 1024, "fp16", 55, False, sigma_qk=3.0),
+], ids=lambda w: w.name)
+def test_both_kernels_agree(oracle, w, monkeypatch):
+    """The same forward with and without RINGATTN_WIDE=0 (which keeps it on ring_walk_kernel): both against the oracle,
+    and against each other within two units in the last place of the row's largest element (the two kernels move
+    their reference maxima at different times, so the probabilities are rounded at different scales)."""
+    q, k, v = api.make_qkv_bits(w)
+    monkeypatch.delenv("RINGATTN_WIDE", raising=False)
+    out_w, lse_w = forward(w, q, k, v)
+    check_rows(oracle, w, q, k, v, out_w, lse_w, np.arange(w.rows))
+    monkeypatch.setenv("RINGATTN_WIDE", "0")
+    out_b, lse_b = forward(w, q, k, v)
+    check_rows(oracle, w, q, k, v, out_b, lse_b, np.arange(w.rows))
+    a, b = out_w.double().cpu().numpy().reshape(-1, w.dim), out_b.double().cpu().numpy().reshape(-1, w.dim)
+    big = np.maximum(np.abs(a), np.abs(b)).max(axis=1, keepdims=True)
+    mant = 10 if w.dtype == "fp16" else 7
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(big, 2.0 ** -14))) - mant)
+    assert (np.abs(a - b) <= 2 * ulp).all()
+    assert np.abs(lse_w.double().cpu().numpy() - lse_b.double().cpu().numpy()).max() <= 1e-4
+
+
+def test_wide_kernel_with_grouped_heads_and_unequal_ranks(oracle):
+    """Shapes the kernel takes beyond plain equal chunks: grouped-query heads and ranks of different lengths
+    (multiples of 32, at least 128).  (The zigzag layout at d = 128 is covered by test_gpu_parity.test_zigzag_layout.)"""
+    # grouped-query heads
+    w = Workload("w_gqa", 1, 4, 128, 4, 512, "bf16", 61, True)
+    q, k, v = api.make_qkv_bits(w)
+    k, v = k[:, :2].copy(), v[:, :2].copy()
+    plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, kv_heads=2)
+    try:
+        out, lse = plan.forward(*(api.bits_to_tensor(x, w.dtype) for x in (q, k, v)))
+        torch.cuda.synchronize()
+    finally:
+        plan.close()
+    k_full, v_full = np.repeat(k, 2, axis=1), np.repeat(v, 2, axis=1)
+    check_rows(oracle, w, q, k_full, v_full, out, lse, np.arange(w.rows))
+    # ranks of different lengths
+    seqlen = (512, 128, 384, 160)
+    S = sum(seqlen)
+    wu = Workload("w_uneq", 1, 2, 128, 1, S, "fp16", 62, True)
+    q, k, v = api.make_qkv_bits(wu)
+    plan = api.RingAttention(len(seqlen), list(seqlen), 128, 1, 2, "fp16", True)
+    try:
+        out, lse = plan.forward(*(api.bits_to_tensor(x, "fp16") for x in (q, k, v)))
+        torch.cuda.synchronize()
+    finally:
+        plan.close()
+    check_rows(oracle, wu, q, k, v, out, lse, np.arange(wu.rows))

@@ -97,3 +97,22 @@ def test_walk_kernel_runs_two_waves_per_simd_without_spills(tmp_path):
                 # taken before the stores, which puts it on a side path of the loop)
                 assert sum(i.startswith("s_barrier") for i in ins) in ((2,) if carried else (1, 2)), (n, lab)
                 assert not any(i.startswith("scratch_") for i in ins), (n, lab)
+
+
+def test_walk64_kernel_runs_one_wave_per_simd(tmp_path):
+    """ring_walk64_kernel (64 query rows per wave) is laid out for one wave per SIMD: more than 256 registers, the two
+    eight-tile rings plus the chunk list in LDS, and next to no scratch (none inside the hand-scheduled loop, which
+    is inline assembly)."""
+    asm, usage = compile_to_asm("ringattn_walk64.hip", tmp_path / "walk64.s")
+    kernels = {n: u for n, u in usage.items() if "ring_walk64_kernel" in n}
+    assert len(kernels) == 2                                  # fp16, bf16
+    for n, u in kernels.items():
+        assert u["Occupancy [waves/SIMD]"] == 1, (n, u)
+        assert u["LDS Size [bytes/block]"] == 2 * 8 * 8192 + 8 * (64 + 2), (n, u)
+        assert u["ScratchSize [bytes/lane]"] <= 128, (n, u)   # the plain-code path of waves with a single score tile
+        start = asm.index("\n" + n + ":")
+        body = asm[start:asm.index(".amdhsa_kernel " + n, start)]
+        blocks = body.split(";;#ASMSTART")[1:]
+        loop = max((b.split(";;#ASMEND")[0] for b in blocks), key=len)
+        assert loop.count("v_mfma_f32_32x32x16") >= 8 * 32    # eight unrolled iterations of 32 MFMAs, and the tails
+        assert "scratch_" not in loop
