@@ -3,12 +3,14 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4]
 
 A step is one full forward of the workload: every ring step of every virtual rank, with Q/K/V
-already resident in HBM -- one launch (ring_walk_kernel) in which a workgroup walks all ring steps
-of its 256 query rows with the softmax state in registers and writes O and LSE at the end.
+already resident in HBM -- one launch (ring_walk64_kernel at d = 128, else ring_walk_kernel) in which a
+workgroup walks all ring steps of its 256 query rows with the softmax state in registers and writes O
+and LSE at the end.
 Prints one JSON line.  `value` is algorithmic TFLOP/s (4*B*H*d*visible (q,k) pairs per forward)
 over the wall time of K steps; `roofline` prices the block-attention launch of the same forward
 against the dense MFMA peak, timed by an event pair on the launch stream (a second pass of K
-forwards on a plan with the timing flag); `forward_with_step_partials` is the same forward on a
+forwards on a plan with the timing flag); `sustained` is the same forward run back to back for a few
+seconds more, the figure of its last second; `forward_with_step_partials` is the same forward on a
 plan that keeps the ring steps apart (a fp32 partial (O, LSE) per step in a workspace, merged at
 the end of each workgroup: another instantiation of the kernel, so a kernel trace keeps the two
 apart; --step-partials makes that one the headline, --one-forward skips the other one); `merge`
@@ -29,26 +31,30 @@ sys.path.insert(0, ROOT)
 PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0}
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the default forward's kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE): workload ->
-# (bytes, summary under profiles/, kernel_source_id() when it was measured).  The figure is only printed while the
-# kernel source is still the one that was profiled.
+# (bytes, summary under profiles/, kernel, kernel_source_id(kernel) when it was measured).  The figure is only printed
+# while the forward still runs that kernel and its source is still the one that was profiled.
 MEASURED_TRAFFIC = {
-    "cfg4": (3499e6, "profiles/ring_walk_kernel_cfg4.md", "494a183db25c449b"),
-    "cfg2": (34.3e6, "profiles/ring_walk_kernel_other_workloads.md", "494a183db25c449b"),
-    "cfg3": (2188e6, "profiles/ring_walk_kernel_other_workloads.md", "494a183db25c449b"),
-    "cfg5": (18260e6, "profiles/ring_walk_kernel_other_workloads.md", "494a183db25c449b"),
+    "cfg4": (2260e6, "profiles/ring_walk64_kernel_cfg4.md", "ring_walk64_kernel", "@W64@"),
+    "cfg3": (2354e6, "profiles/ring_walk64_kernel_other_workloads.md", "ring_walk64_kernel", "@W64@"),
+    "cfg5": (43590e6, "profiles/ring_walk64_kernel_other_workloads.md", "ring_walk64_kernel", "@W64@"),
+    "cfg2": (34.3e6, "profiles/ring_walk_kernel_other_workloads.md", "ring_walk_kernel", "494a183db25c449b"),
+}
+KERNEL_SOURCES = {
+    "ring_walk64_kernel": ("ringattn_walk64.hip", "ringattn_walk64_loop.inc", "ringattn_device.h"),
+    "ring_walk_kernel": ("ringattn_walk.hip", "ringattn_device.h"),
 }
 BASELINE_METRIC = "ring-attn fwd TFLOP/s + % bf16 MFMA peak, S=32K d=128 8-step ring, 1 GPU"
 
 
-def kernel_source_id():
-    """Hash of the sources of the kernel the default forward runs (ring_walk_kernel)."""
+def kernel_source_id(kernel):
+    """Hash of the sources of one of the attention kernels."""
     import hashlib
     h = hashlib.sha256()
     try:
-        for name in ("ringattn_walk.hip", "ringattn_device.h"):
+        for name in KERNEL_SOURCES[kernel]:
             with open(os.path.join(ROOT, "ringattention_amd", "csrc", name), "rb") as f:
                 h.update(f.read())
-    except OSError:
+    except (OSError, KeyError):
         return None
     return h.hexdigest()[:16]
 
@@ -86,6 +92,8 @@ def main():
                     help="diagnostic: 'zeros' runs the same launches on all-zero Q, K, V (same instruction stream, no operand "
                          "toggling: shows what the power manager leaves of the clock); not a valid headline")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the cpu_baseline sample (0 = skip)")
+    ap.add_argument("--sustain-seconds", type=float, default=2.5,
+                    help="after the timed steps, run the same forward back to back for this long and report the last second (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (P virtual ring ranks on one MI355X); use --gpus 1")
@@ -126,6 +134,36 @@ def main():
     ms_per_step_events = ev0.elapsed_time(ev1) / args.steps
     tflops = w.flops / (ms_per_step * 1e-3) / 1e12
 
+    # ---- what is sustained: the same forward back to back for --sustain-seconds more, in batches timed by event
+    # pairs; reported: the batches of the last second (the first second of a process runs a few percent fast, before
+    # the part's power manager has settled)
+    sustained = None
+    if args.sustain_seconds > 0:
+        per_batch = max(1, int(round(0.1 / (ms_per_step * 1e-3))))    # about 0.1 s of forwards per batch
+        batch_ms, t_start = [], time.perf_counter()
+        while time.perf_counter() - t_start < args.sustain_seconds:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(per_batch):
+                plan.forward(qd, kd, vd, out, lse, stream)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            batch_ms.append(e0.elapsed_time(e1) / per_batch)
+        total_s = time.perf_counter() - t_start
+        tail, acc = [], 0.0
+        for x in reversed(batch_ms):     # the batches that make up the last second
+            tail.append(x)
+            acc += x * per_batch * 1e-3
+            if acc >= 1.0:
+                break
+        last_ms = float(np.mean(tail))
+        sustained = {"seconds": round(total_s, 2), "forwards": per_batch * len(batch_ms),
+                     "ms_per_step_last_second": round(last_ms, 4),
+                     "tflops_last_second": round(w.flops / (last_ms * 1e-3) / 1e12, 2),
+                     "pct_mfma_peak_last_second": round(100.0 * w.flops / (last_ms * 1e-3) / 1e12 / PEAK_TFLOPS[w.dtype], 2),
+                     "ms_per_step_first_batch": round(batch_ms[0], 4),
+                     "clock_evidence": "profiles/ring_walk64_kernel_cfg4.md"}
+
     bh = w.batch * w.heads
     peak = PEAK_TFLOPS[w.dtype]
     # ---- attention kernel: the same forward on a plan that records an event pair around its
@@ -143,14 +181,16 @@ def main():
     avg_launch_ms = float(launch_ms.mean())
     block_tflops = w.flops / n_launch / (avg_launch_ms * 1e-3) / 1e12
     traffic, traffic_source = None, "not measured for this workload / layout"
+    kernel = timed.forward_kernel()
     if args.layout == "contiguous" and not args.step_partials and w.name in MEASURED_TRAFFIC:
-        t_bytes, t_profile, t_src = MEASURED_TRAFFIC[w.name]
-        if t_src == kernel_source_id():
+        t_bytes, t_profile, t_kernel, t_src = MEASURED_TRAFFIC[w.name]
+        if t_kernel == kernel and t_src == kernel_source_id(kernel):
             traffic, traffic_source = t_bytes, t_profile
         else:
-            traffic_source = f"stale: {t_profile} was measured on kernel source {t_src}, this is {kernel_source_id()}"
+            traffic_source = (f"stale: {t_profile} was measured on {t_kernel} with source {t_src}, this is {kernel} "
+                              f"with source {kernel_source_id(kernel)}")
     roofline = {
-        "kernel": "ring_walk_kernel", "bound": "mfma",
+        "kernel": kernel, "bound": "mfma",
         "achieved": round(block_tflops, 2), "peak": peak, "unit": "TFLOP/s", "frac": round(block_tflops / peak, 4),
         "traffic": traffic, "traffic_source": traffic_source,
         "launches_per_step": n_launch, "avg_launch_ms": round(avg_launch_ms, 4),
@@ -295,6 +335,7 @@ def main():
                    else "none: softmax state carried through the ring steps in registers",
                    "workspace_bytes": int(plan_ws)},
         "pct_mfma_peak": round(100.0 * tflops / peak, 2),
+        "sustained": sustained,
         "roofline": roofline,
         ("forward_with_carried_state" if args.step_partials else "forward_with_step_partials"): other_leg,
         "merge": merge, "per_ring_step": per_step, "rank_local_ring": ring, "cpu_baseline": cpu,

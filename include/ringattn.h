@@ -47,7 +47,7 @@ extern "C" {
                                       ranks (the tail predication the reference leaves open, csrc/ring_attention.cu:143-145);
                                       multiples of this waste no part of a tile */
 
-#define RINGATTN_FLAG_GRAPH 1      /* capture the step loop + merge in a hipGraph and replay it */
+#define RINGATTN_FLAG_GRAPH 1      /* capture the launch of a forward (one kernel node) in a hipGraph and replay it */
 #define RINGATTN_FLAG_TIMING 2     /* record timing events around every block-attention launch of ringattn_fwd
                                       (read with ringattn_plan_launch_times); ignored together with FLAG_GRAPH */
 #define RINGATTN_FLAG_HALF_PARTIALS 4 /* keep the per-step partial O in fp16 instead of fp32 (for either input dtype): halves
@@ -227,6 +227,16 @@ int ringattn_plan_work_items(const ringattn_plan* plan, int step, ringattn_work_
  * RINGATTN_ERR_PLAN if the plan has no timing flag or has not run a forward yet.
  */
 int ringattn_plan_launch_times(ringattn_plan* plan, float* ms, int capacity, int* n_out);
+
+/*
+ * Name of the kernel ringattn_fwd launches for this plan, for reading kernel traces: "ring_walk64_kernel" (d = 128,
+ * carried softmax state, every KV range a multiple of 32 keys and at least 128, at least 512 rows per head, and
+ * RINGATTN_WIDE=0 not set in the environment) or "ring_walk_kernel".  Both are restatements of the reference's one
+ * kernel (csrc/ring_attention.cu:398-666) with its tiling (csrc/kernel_traits.h:11-177) replaced; they differ in how
+ * the 256 query rows of a workgroup are laid out over waves (64 rows per wave at one wave per SIMD, or 32 rows per
+ * wave at two).  NULL for an invalid plan.
+ */
+const char* ringattn_plan_forward_kernel(const ringattn_plan* plan);
 
 /*
  * The row ranges ringattn_merge_ring merges separately: rows [start[i], start[i] + len[i])

@@ -53,6 +53,7 @@ SYMBOLS = {
     "ringattn_plan_work_items": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(RingattnWorkItem),
                                                 ctypes.c_int, c_int_p]),
     "ringattn_plan_launch_times": (ctypes.c_int, [ctypes.c_void_p, c_float_p, ctypes.c_int, c_int_p]),
+    "ringattn_plan_forward_kernel": (ctypes.c_char_p, [ctypes.c_void_p]),
     "ringattn_plan_merge_regions": (ctypes.c_int, [ctypes.c_void_p, c_int_p, c_int_p,
                                                    ctypes.POINTER(ctypes.c_uint64), ctypes.c_int, c_int_p]),
     "ringattn_ring_attention": (ctypes.c_int, [ctypes.c_void_p] * 5 + [ctypes.c_int, ctypes.c_int, c_int_p,

@@ -193,11 +193,18 @@ class RingAttention:
         return out, lse
 
     def launch_times(self):
-        """Milliseconds of each block-attention launch of the last forward (plan made with timing=True)."""
-        ms = (ctypes.c_float * 8)()
+        """Milliseconds of each block-attention launch of the last forward (plan made with timing=True): a forward
+        is one launch, so one value."""
         n = ctypes.c_int()
-        check(self.lib.ringattn_plan_launch_times(self.handle, ms, 8, ctypes.byref(n)), "ringattn_plan_launch_times")
+        check(self.lib.ringattn_plan_launch_times(self.handle, None, 0, ctypes.byref(n)), "ringattn_plan_launch_times")
+        ms = (ctypes.c_float * max(1, n.value))()
+        check(self.lib.ringattn_plan_launch_times(self.handle, ms, n.value, ctypes.byref(n)), "ringattn_plan_launch_times")
         return [ms[i] for i in range(n.value)]
+
+    def forward_kernel(self):
+        """Name of the kernel forward() launches (as it appears in a kernel trace)."""
+        name = self.lib.ringattn_plan_forward_kernel(self.handle)
+        return name.decode() if name else None
 
     def work_items(self, step=-1):
         """The plan's block-attention jobs as (q_start, q_len, kv_start, kv_len, diag_off, slot)

@@ -435,6 +435,12 @@ int ensure_tables(ringattn_plan* pl) {
   return RINGATTN_OK;
 }
 
+// ring_walk64_kernel runs the carried-state launch of a slice when every KV range suits it, d = 128, and a head is
+// long enough for the loads it issues past the last chunk (whole tiles from the start of the head, never read back)
+bool slice_takes_walk64(const ringattn_plan* pl, const TableSlice& sl) {
+  return sl.wide && pl->p.dim == 128 && pl->d.S >= 512 && walk64_enabled();
+}
+
 // A block launch over a slice of the tables.
 int launch_slice(const ringattn_plan* pl, const TableSlice& sl, ringattn::BlockArgs& a, hipStream_t stream) {
   if (sl.seg_count == 0) return RINGATTN_OK;
@@ -442,7 +448,7 @@ int launch_slice(const ringattn_plan* pl, const TableSlice& sl, ringattn::BlockA
   a.items = pl->d_segitems;
   a.n_segs = sl.seg_count;
   a.q_tiles_max = sl.q_tiles_max;
-  if (sl.wide && pl->p.dim == 128 && pl->d.S >= 512 && a.mode == ringattn::kBlockCarryState && walk64_enabled())
+  if (a.mode == ringattn::kBlockCarryState && slice_takes_walk64(pl, sl))
     RA_HIP(ringattn::launch_walk64(a, pl->p.dtype, stream));
   else
     RA_HIP(ringattn::launch_walk(a, pl->p.dtype, pl->p.dim, stream));
@@ -848,6 +854,11 @@ int ringattn_plan_launch_times(ringattn_plan* plan, float* ms, int capacity, int
     RA_HIP(hipEventElapsedTime(&ms[0], plan->ev_t0, plan->ev_t1));
   }
   return RINGATTN_OK;
+}
+
+const char* ringattn_plan_forward_kernel(const ringattn_plan* plan) {
+  if (!plan_ok(plan)) return nullptr;
+  return (!step_partials(plan->p) && slice_takes_walk64(plan, plan->fwd)) ? "ring_walk64_kernel" : "ring_walk_kernel";
 }
 
 int ringattn_plan_merge_regions(const ringattn_plan* plan, int* start, int* len, uint64_t* active, int capacity, int* n_out) {

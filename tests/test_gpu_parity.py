@@ -5,7 +5,7 @@ inputs.  Tolerances are the ones the engine is specified with:
     LSE : relative error <= 1e-3 (fp32)
 
 Large workloads are compared on whole heads (cfg2 in full; one or two complete heads of cfg3 and
-cfg4; complete q tiles at chunk starts, middles and ends of cfg5) plus a seeded sample of rows
+cfg4; complete 256-row q tiles at chunk starts, middles and ends of cfg5) plus a seeded sample of rows
 (the first rows of the sequence, where causal rows see few keys and |O| is largest, are always
 included), and through size-independent properties on the full output.  Where the roundings that
 the algorithm prescribes (the store of O and the probabilities of the PV product, both in the storage
@@ -59,7 +59,7 @@ def storage_ulp(x, dtype):
     return 2.0 ** (e - mant)
 
 
-def check_rows(oracle, w, q, k, v, out, lse, rows, scale=None, half_partials=None):
+def check_rows(oracle, w, q, k, v, out, lse, rows, scale=None, half_partials=None, plain_bound=None):
     """O against the float64 oracle: max-abs error <= 1e-2 -- or, where that is more, what the two roundings
     that the algorithm prescribes allow at that element: half a unit in the last place of the storage type for
     the store of O (csrc/ring_attention.cu:635; a bf16 value in [4, 8) is a multiple of 2^-5, so even the
@@ -73,7 +73,12 @@ def check_rows(oracle, w, q, k, v, out, lse, rows, scale=None, half_partials=Non
     oracle rounded to the storage type (two with fp16 per-step partials), except that one row in a thousand
     may use u max|V| plus half an ulp for the store instead (rows whose few dominant keys carry large V
     entries that nearly cancel).
-    LSE: relative error <= 1e-3."""
+    LSE: relative error <= 1e-3.
+    plain_bound: the rounding allowance for the probabilities may not be used at all -- every element within
+    max(1e-2, half an ulp of the storage type).  Always so for fp16 (half an ulp of fp16 stays below 1e-2 up to
+    |O| = 16, and its probabilities carry 2^-11, not 2^-8); the five specified workloads ask for it explicitly."""
+    if plain_bound is None:
+        plain_bound = w.dtype == "fp16"
     o_ref, l_ref = oracle.attention_rows(q, k, v, w.dtype, causal=w.causal, rows=rows, scale=scale)
     idx = torch.from_numpy(rows).cuda()
     o_gpu = out.reshape(-1, w.dim)[idx].double().cpu().numpy()
@@ -86,12 +91,15 @@ def check_rows(oracle, w, q, k, v, out, lse, rows, scale=None, half_partials=Non
     p_round = u_p * v_max
     err = np.abs(o_gpu - o_ref)
     beyond = np.unique(np.nonzero(err > tol)[0])
-    if len(beyond):  # rows with an element beyond the plain bound: what do their own roundings allow?
+    if len(beyond) and not plain_bound:  # rows with an element beyond the plain bound: what do their own roundings allow?
         v_abs = (np.ascontiguousarray(v).view(np.uint16) & 0x7FFF).view(v.dtype)
         mean_abs_v, _ = oracle.attention_rows(q, k, v_abs, w.dtype, causal=w.causal, rows=rows[beyond], scale=scale)
         tol[beyond] = np.maximum(tol[beyond], 0.5 * ulp[beyond] + u_p * mean_abs_v)
         print(f"parity {w.name}: {len(beyond)} of {len(rows)} rows have an element beyond max(1e-2, half an ulp); "
               f"their own rounding bound is up to {tol[beyond].max():.3e}")
+        # the allowance is for rows that average very few V rows (the first rows of a causal sequence, a softmax
+        # peaked by huge logits), never for a workload at large: at most two rows in a hundred
+        assert len(beyond) <= max(4, len(rows) // 50), f"{w.name}: {len(beyond)} rows beyond the plain bound"
     err_o = err.max()
     err_l = (np.abs(l_gpu - l_ref) / np.maximum(np.abs(l_ref), 1e-3)).max()
     # also against the oracle rounded to the storage type (what a perfect kernel would store)
@@ -104,7 +112,8 @@ def check_rows(oracle, w, q, k, v, out, lse, rows, scale=None, half_partials=Non
     ulp_r = storage_ulp(np.maximum(np.abs(o_gpu), np.abs(o_rounded)).max(axis=1, keepdims=True), w.dtype)
     print(f"parity {w.name}: {len(rows)} rows, max|dO| = {err_o:.3e} vs fp64, {err_r.max():.3e} vs rounded fp64 "
           f"({(err_r / ulp_r).max():.2f} ulp), max rel dLSE = {err_l:.3e}, max|O| = {np.abs(o_ref).max():.2f}, "
-          f"{int((tol > O_TOL).sum())} elements where half an ulp exceeds 1e-2")
+          f"{int((tol > O_TOL).sum())} elements where half an ulp exceeds 1e-2, "
+          f"bound: {'max(1e-2, half an ulp), no allowance' if plain_bound else 'with the rounding allowance'}")
     assert (err <= tol).all(), f"{w.name}: max|dO| = {err_o:.3e}, worst excess {(err - tol).max():.3e}"
     # fp16 per-step partials (RINGATTN_FLAG_HALF_PARTIALS) round once more on the way: two units then
     ulps = 2 if (w.half_partials if half_partials is None else half_partials) else 1
@@ -127,7 +136,7 @@ def whole_head_rows(w, heads):
 
 def workload_rows(w):
     """Rows compared for each of the five workloads: whole heads where the oracle gets through them
-    in seconds, complete 128-row q tiles at the start, middle and end of chunks for the longest one,
+    in seconds, complete 256-row q tiles (a workgroup's rows) at the start, middle and end of chunks for the longest one,
     plus the seeded sample (first rows of the sequence, last head, chunk edges)."""
     bh = w.batch * w.heads
     if w.name == "cfg2":
@@ -138,10 +147,10 @@ def workload_rows(w):
         rows = np.concatenate([whole_head_rows(w, [0, bh - 1]), sample_rows(w, 384)])
     elif w.name == "cfg5":
         tiles = []
-        for head, chunk, where in ((0, 0, 0), (0, 3, w.chunk // 2), (5, 7, w.chunk - 128), (bh - 1, w.npes - 1, w.chunk - 128),
-                                   (bh - 1, 8, 0), (9, 15, 4096 + 128)):
+        for head, chunk, where in ((0, 0, 0), (0, 3, w.chunk // 2), (5, 7, w.chunk - 256), (bh - 1, w.npes - 1, w.chunk - 256),
+                                   (bh - 1, 8, 0), (9, 15, 4096 + 256)):
             first = head * w.seq + chunk * w.chunk + where
-            tiles.append(np.arange(first, first + 128))
+            tiles.append(np.arange(first, first + 256))
         rows = np.concatenate(tiles + [sample_rows(w, 1400)])
     else:
         rows = sample_rows(w, 256)
@@ -152,7 +161,7 @@ def test_cfg1_full_against_oracle_and_golden(oracle):
     w = WORKLOADS["cfg1"]
     q, k, v = api.make_qkv_bits(w)
     out, lse = forward(w, q, k, v)
-    check_rows(oracle, w, q, k, v, out, lse, np.arange(w.rows))
+    check_rows(oracle, w, q, k, v, out, lse, np.arange(w.rows), plain_bound=True)
     g = np.load(os.path.join(GOLD, "cfg1_expected.npz"))   # torch-library fixture, independent of the oracle
     assert np.abs(out.float().cpu().numpy() - g["o_f32"]).max() <= O_TOL
     assert np.abs(lse.double().cpu().numpy() - g["lse_f64"]).max() <= LSE_RTOL * np.abs(g["lse_f64"]).max()
@@ -168,14 +177,16 @@ def test_causal_small_golden(oracle):
 
 
 @pytest.mark.parametrize("name,step_partials", [("cfg2", False), ("cfg2", True), ("cfg3", False), ("cfg3", True),
-                                                ("cfg4", False), ("cfg4", True), ("cfg5", False)])
+                                                ("cfg4", False), ("cfg4", True), ("cfg5", False), ("cfg5", True)])
 def test_workload_whole_heads(oracle, name, step_partials):
     # step_partials: the forward that keeps the ring steps apart (per-step partials in the workspace,
     # fp16 where the workload says so) instead of carrying the softmax state through them
     w = WORKLOADS[name]
     q, k, v = api.make_qkv_bits(w)
     out, lse = forward(w, q, k, v, step_partials=step_partials)
-    check_rows(oracle, w, q, k, v, out, lse, workload_rows(w), half_partials=w.half_partials and step_partials)
+    # the five specified workloads: max(1e-2, half an ulp of the storage type) for every element, no allowance
+    check_rows(oracle, w, q, k, v, out, lse, workload_rows(w), half_partials=w.half_partials and step_partials,
+               plain_bound=True)
     # full-size properties: finite everywhere, convexity |O| <= max|V| (O is an average of V rows)
     assert torch.isfinite(out).all() and torch.isfinite(lse).all()
     vmax = np.abs(bits_to_float64(v, w.dtype)).max()
@@ -259,7 +270,7 @@ def test_unequal_rank_lengths(oracle, seqlen, causal, d, dtype):
     ((640, 384, 896), False, 64, "bf16", "contiguous"),    # whole key tiles, chunk lengths that are no multiples of four tiles
 ])
 def test_ragged_lengths(oracle, seqlen, causal, d, dtype, layout):
-    # lengths that are no multiples of the 128-row q tile or the 32-key tile: the tail
+    # lengths that are no multiples of the 256-row q tile or the 32-key tile: the tail
     # predication the reference leaves open (csrc/ring_attention.cu:143-145)
     P, S, B, H = len(seqlen), sum(seqlen), 2, 2
     w = Workload("ragged", B, H, d, 1, S, dtype, 95, causal)
