@@ -271,8 +271,13 @@ int ringattn_ring_attention(const void* q, const void* k, const void* v, void* o
  * in a per-call allocation, lives in a static device array of ringattn_noalloc_scratch_bytes()
  * bytes (4 KiB, held by every GPU the library runs on until the process ends): enough for
  * RINGATTN_MAX_NPES steps, and a ring with more ranks is refused with RINGATTN_ERR_NPES like
- * everywhere else.  All calls on one GPU share that array: calls that overlap on one GPU (two
- * streams, two threads) race; nothing in it needs clearing between calls.
+ * everywhere else.  All calls on one GPU share that array.  A call's table takes the next slice of it, round
+ * robin, and the attention kernel reads its slice for as long as it runs: calls on one stream are ordered by the
+ * stream, and calls on several streams or threads may overlap as long as no more of them are in flight on a GPU
+ * than slices fit (fourteen with 8-step rings, 288 bytes each; one when a table takes more than half the array).
+ * Beyond that a running kernel may find another call's KV ranges in its table and read outside its K and V: do
+ * not let that many calls overlap.  Nothing in the array needs clearing between calls.  The first call on a
+ * device looks up the array's address (hipGetSymbolAddress): make it outside a stream capture.
  */
 int ringattn_ring_attention_noalloc(const void* q, const void* k, const void* v, void* out, float* lse,
                                     int npes, int mype, const int* seqlen, int dim, int max_seq,

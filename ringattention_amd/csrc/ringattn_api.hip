@@ -593,6 +593,10 @@ int run_rank_call(const RankCall& rc, void* scratch, const void* q, const void* 
 // Static device scratch of ringattn_ring_attention_noalloc.  In host code the array's name is
 // only a handle for hipGetSymbolAddress; the device address is looked up once per device
 // (each GPU holds its own copy of the array) and kept.
+// A call's table (32 bytes + 32 per visible ring step) takes the next slice of the array, round robin: the walk
+// kernel reads its table for as long as it runs, so a later call must not overwrite it while an earlier one is still
+// in flight on another stream.  With the tables of an 8-step ring (288 bytes) fourteen calls can be in flight
+// before a slice is used again; a call whose table needs more than half the array has it to itself.
 constexpr size_t kScratchBytes = 4096;
 static_assert(kScratchBytes >= sizeof(ringattn::Segment) + RINGATTN_MAX_NPES * sizeof(ringattn::SegItem),
               "the table of the largest ring fits");
@@ -600,11 +604,13 @@ static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mu;
 void* g_scratch_ptr[kMaxDevices] = {};
+size_t g_scratch_next[kMaxDevices] = {};
 
-int device_scratch(void** base) {
+int device_scratch(size_t bytes, void** slice) {
   int dev = -1;
   RA_HIP(hipGetDevice(&dev));
   if (dev < 0 || dev >= kMaxDevices) return RINGATTN_ERR_SHAPE;
+  if (bytes > kScratchBytes) return RINGATTN_ERR_WORKSPACE;
   std::lock_guard<std::mutex> lk(g_scratch_mu);
   if (!g_scratch_ptr[dev]) {
     void* ptr = nullptr;
@@ -612,7 +618,10 @@ int device_scratch(void** base) {
     if (!ptr) return RINGATTN_ERR_HIP;
     g_scratch_ptr[dev] = ptr;
   }
-  *base = g_scratch_ptr[dev];
+  const size_t need = (bytes + 31) & ~(size_t)31;   // tables are read with 16-byte scalar loads
+  if (g_scratch_next[dev] + need > kScratchBytes) g_scratch_next[dev] = 0;
+  *slice = (char*)g_scratch_ptr[dev] + g_scratch_next[dev];
+  g_scratch_next[dev] += need;
   return RINGATTN_OK;
 }
 
@@ -928,11 +937,10 @@ int ringattn_ring_attention_noalloc(const void* q, const void* k, const void* v,
   RankCall rc_;
   int rc = prepare_rank_call(&rc_, q, k, v, out, npes, mype, seqlen, dim, max_seq, dtype, causal, softmax_scale);
   if (rc != RINGATTN_OK) return rc;
-  if (rc_.scratch_bytes > kScratchBytes) return RINGATTN_ERR_WORKSPACE;
-  void* base = nullptr;
-  rc = device_scratch(&base);
+  void* slice = nullptr;
+  rc = device_scratch(rc_.scratch_bytes, &slice);
   if (rc != RINGATTN_OK) return rc;
-  return run_rank_call(rc_, base, q, k, v, out, lse, (hipStream_t)stream);
+  return run_rank_call(rc_, slice, q, k, v, out, lse, (hipStream_t)stream);
 }
 
 const char* ringattn_strerror(int code) {

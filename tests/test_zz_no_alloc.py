@@ -65,3 +65,56 @@ def test_noalloc_entry_limits():
     with pytest.raises(_lib.RingattnError) as e:
         api.ring_attention_noalloc(q, kv, kv, torch.empty_like(q), npes, 0, [c] * npes, dim, c)
     assert e.value.code == 2              # RINGATTN_ERR_NPES
+
+
+def test_noalloc_entry_under_stream_capture_allocates_nothing():
+    """What the entry is for: a caller that records it into a graph.  After one warm call outside the capture (the
+    first call on a device looks up the scratch address), the call is captured on a side stream -- an allocation, a
+    host copy or a synchronisation inside it would fail the capture --, the graph is replayed twice with eager work
+    in between, and every replay gives the bits of the allocating entry point."""
+    seqlen, dim, mype, npes = [512, 384, 512], 128, 2, 3
+    g = torch.Generator(device="cpu").manual_seed(11)
+    k = torch.randn(sum(seqlen), dim, generator=g).bfloat16().cuda()
+    v = torch.randn(sum(seqlen), dim, generator=g).bfloat16().cuda()
+    q = torch.randn(seqlen[mype], dim, generator=g).bfloat16().cuda()
+    ref, out = torch.empty_like(q), torch.empty_like(q)
+    lse_ref = torch.empty(seqlen[mype], dtype=torch.float32, device="cuda")
+    lse = torch.empty_like(lse_ref)
+    api.ring_attention(q, k, v, ref, npes, mype, seqlen, dim, max(seqlen), lse=lse_ref, causal=True)
+    api.ring_attention_noalloc(q, k, v, out, npes, mype, seqlen, dim, max(seqlen), lse=lse, causal=True)   # warm
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        api.ring_attention_noalloc(q, k, v, out, npes, mype, seqlen, dim, max(seqlen), lse=lse, causal=True, stream=side)
+    for _ in range(2):
+        out.fill_(5.0)
+        lse.fill_(5.0)
+        (k.float() @ v.float().t()).sum().item()      # the program's own eager work and a synchronisation in between
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+        assert torch.equal(lse.view(torch.int32), lse_ref.view(torch.int32))
+
+
+def test_noalloc_calls_in_flight_on_several_streams():
+    """Each call's table takes its own slice of the scratch, so a handful of calls may be in flight at once."""
+    dim, npes = 128, 4
+    seqlen = [1024] * npes
+    gen = torch.Generator(device="cpu").manual_seed(12)
+    k = torch.randn(sum(seqlen), dim, generator=gen).half().cuda()
+    v = torch.randn(sum(seqlen), dim, generator=gen).half().cuda()
+    qs = [torch.randn(1024, dim, generator=gen).half().cuda() for _ in range(npes)]
+    refs = [torch.empty_like(x) for x in qs]
+    outs = [torch.empty_like(x) for x in qs]
+    for r in range(npes):
+        api.ring_attention(qs[r], k, v, refs[r], npes, r, seqlen, dim, 1024, causal=True)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(npes)]
+    for rep in range(3):
+        for r in range(npes):
+            api.ring_attention_noalloc(qs[r], k, v, outs[r], npes, r, seqlen, dim, 1024, causal=True, stream=streams[r])
+    for s in streams:
+        s.synchronize()
+    for r in range(npes):
+        assert torch.equal(outs[r].view(torch.int16), refs[r].view(torch.int16)), r
