@@ -258,6 +258,23 @@ def main():
         per_step = {"ms": [round(float(x), 4) for x in step_ms],
                     "tflops": [round(f / (t * 1e-3) / 1e12, 1) for f, t in zip(step_flops, step_ms)]}
     del o_parts, l_parts
+    # the same merge with a row's steps next to each other (RINGATTN_FLAG_ROW_PARTIALS): same bytes, one run per row
+    rowp = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, graph=False, layout=args.layout,
+                             half_partials=w.half_partials, row_partials=True)
+    o_shape, l_shape = rowp.parts_shapes()
+    o_parts = torch.empty(o_shape, dtype=rowp.part_dtype, device="cuda").normal_()
+    l_parts = torch.empty(l_shape, dtype=torch.float32, device="cuda").normal_()
+    rowp.merge_ring(o_parts, l_parts, out, lse, stream)
+    for r in range(reps):
+        ev[r].record(stream)
+        rowp.merge_ring(o_parts, l_parts, out, lse, stream)
+    ev[reps].record(stream)
+    torch.cuda.synchronize()
+    row_ms = float(np.mean([ev[r].elapsed_time(ev[r + 1]) for r in range(reps)]))
+    merge["row_major_partials"] = {"achieved": round(merge_bytes / (row_ms * 1e-3) / 1e9, 1), "ms": round(row_ms, 4),
+                                   "frac": round(merge_bytes / (row_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+    rowp.close()
+    del o_parts, l_parts
 
     # ---- optional: the ring as one process per GPU would run it, replayed rank by rank on this
     # GPU with rank-local buffers (ringattn_rank_step_fwd / ringattn_rank_merge): every launch is one

@@ -61,6 +61,14 @@ extern "C" {
                                       ringattn_merge_ring, bit for bit, in one launch.  Without the flag (the default)
                                       the softmax state (max, sum, acc-O) runs through all steps in registers, as in the
                                       reference's kernel (csrc/ring_attention.cu:439-443,597), and no workspace is needed */
+#define RINGATTN_FLAG_ROW_PARTIALS 16 /* caller-held per-step partials keep a row's steps next to each other:
+                                      o_parts [batch*heads*S, npes, dim] and lse_parts [batch*heads*S, npes] instead of
+                                      [npes, batch*heads*S, dim] / [npes, batch*heads*S].  ringattn_block_fwd and
+                                      ringattn_rank_step_fwd then take the BASE of those buffers for every step and
+                                      write entry `step` of each row; ringattn_merge_ring / ringattn_rank_merge read a
+                                      row's steps as one contiguous run (the merge of many short steps -- 32 steps of
+                                      256-byte fp16 rows -- then streams instead of gathering pieces 4 MB apart).  No
+                                      effect on ringattn_fwd */
 
 /*
  * Placement of the sequence on the ranks.  CONTIGUOUS: rank r holds the tokens that follow

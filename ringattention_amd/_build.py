@@ -21,18 +21,41 @@ HIPCC_FLAGS = [
 ]
 
 
+_TOOLCHAIN = None
+
+
+def toolchain_id():
+    """What else a build product depends on: the compile flags, the compiler and (for the torch front end) torch."""
+    global _TOOLCHAIN
+    if _TOOLCHAIN is None:
+        hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+        try:
+            ver = subprocess.run([hipcc, "--version"], capture_output=True, text=True).stdout
+        except OSError:
+            ver = "no hipcc"
+        try:
+            import torch
+            tv = torch.__version__
+        except Exception:
+            tv = "no torch"
+        _TOOLCHAIN = "\n".join(HIPCC_FLAGS) + "\n" + ver + "\n" + tv
+    return _TOOLCHAIN
+
+
 def source_id(paths):
-    """sha256 over the given files: what a build product was made from."""
+    """sha256 over the given files, the compile flags and the toolchain versions: what a build product was made from."""
     import hashlib
     h = hashlib.sha256()
     for path in sorted(paths):
         with open(path, "rb") as f:
             h.update(os.path.basename(path).encode() + b"\0" + f.read())
+    h.update(toolchain_id().encode())
     return h.hexdigest()
 
 
 def library_sources():
     return [os.path.join(CSRC, s) for s in SOURCES] + [os.path.join(CSRC, "ringattn_kernels.h"), os.path.join(CSRC, "ringattn_device.h"),
+                                                       os.path.join(CSRC, "ringattn_walk64_loop.inc"),
                                                        os.path.join(REPO_DIR, "include", "ringattn.h")]
 
 
@@ -52,6 +75,8 @@ def write_stamp(product, sources):
 
 def build_library(verbose=False):
     """Compile every HIP source of the package into libringattn.so.  Always recompiles."""
+    if os.environ.get("RINGATTN_LIB"):
+        raise RuntimeError("RINGATTN_LIB names a library built elsewhere: not overwriting it (unset it to build the package's own)")
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
         raise RuntimeError("hipcc not found: cannot build libringattn.so")

@@ -20,6 +20,7 @@ FLAG_GRAPH = 1
 FLAG_TIMING = 2
 FLAG_HALF_PARTIALS = 4
 FLAG_STEP_PARTIALS = 8
+FLAG_ROW_PARTIALS = 16
 LAYOUT_CODE = {"contiguous": 0, "zigzag": 1}
 
 
@@ -76,7 +77,7 @@ class RingAttention:
 
     def __init__(self, npes, chunk, dim, batch=1, heads=1, dtype="fp16", causal=False, softmax_scale=0.0, graph=False,
                  kv_heads=0, layout="contiguous", timing=False, half_partials=False, workspace=None,
-                 step_partials=False):
+                 step_partials=False, row_partials=False):
         """`chunk`: tokens per rank -- one int for equal chunks or a list of npes lengths
         (the per-PE seqlen[] of csrc/ring_attention.cu:753).  `kv_heads`: heads of K and V for
         grouped-query attention (0 = same as `heads`).  `layout`: "contiguous" (rank r holds
@@ -86,7 +87,10 @@ class RingAttention:
         block_forward + merge_ring) instead of carrying the softmax state through all steps in
         registers.  `half_partials`: keep per-step partial O in fp16 (half the workspace and merge
         traffic; needs |V| < 65504).  `workspace`: a (device address, bytes) pair the caller owns
-        and keeps alive, instead of an allocation by the plan (only a step_partials plan needs one)."""
+        and keeps alive, instead of an allocation by the plan (only a step_partials plan needs one).
+        `row_partials`: caller-held per-step partials are [B, H, S, npes, d] / [B, H, S, npes] (a row's steps next to
+        each other) instead of [npes, B, H, S, d] / [npes, B, H, S]; block_forward / rank_step_forward then take the
+        whole buffers for every step."""
         self.lib = _lib.load()
         self.seqlen = [int(chunk)] * npes if isinstance(chunk, int) else [int(x) for x in chunk]
         if len(self.seqlen) != npes:
@@ -96,12 +100,14 @@ class RingAttention:
         self.torch_dtype = TORCH_DTYPE[self.dtype_code]
         self.causal = bool(causal)
         self.part_dtype = torch.float16 if half_partials else torch.float32
+        self.row_partials = bool(row_partials)
         self.seq = sum(self.seqlen)
         self.kv_heads = kv_heads if kv_heads else heads
         self.params = make_params(npes, self.seqlen, dim, batch, heads, dtype, causal, softmax_scale,
                                   (FLAG_GRAPH if graph else 0) | (FLAG_TIMING if timing else 0)
                                   | (FLAG_HALF_PARTIALS if half_partials else 0)
-                                  | (FLAG_STEP_PARTIALS if step_partials else 0), kv_heads,
+                                  | (FLAG_STEP_PARTIALS if step_partials else 0)
+                                  | (FLAG_ROW_PARTIALS if row_partials else 0), kv_heads,
                                   LAYOUT_CODE[layout])
         self.handle = ctypes.c_void_p()
         ws_ptr, ws_bytes = (None, 0) if workspace is None else (ctypes.c_void_p(int(workspace[0])), int(workspace[1]))
@@ -122,6 +128,20 @@ class RingAttention:
     def _shape(self):
         return (self.batch, self.heads, self.seq, self.dim)
 
+    def parts_shapes(self):
+        """Shapes of caller-held per-step partials (O, LSE) for merge_ring: slot-major, or a row's steps adjacent."""
+        b, h, s, d = self._shape()
+        if self.row_partials:
+            return (b, h, s, self.npes, d), (b, h, s, self.npes)
+        return (self.npes, b, h, s, d), (self.npes, b, h, s)
+
+    def rank_parts_shapes(self, rank):
+        """parts_shapes() for the rank-local calls (rank_step_forward, rank_merge): the rank's rows only."""
+        b, h, rows, d = self.batch, self.heads, self.seqlen[rank], self.dim
+        if self.row_partials:
+            return (b, h, rows, self.npes, d), (b, h, rows, self.npes)
+        return (self.npes, b, h, rows, d), (self.npes, b, h, rows)
+
     def _qkv_specs(self, q, k, v):
         kv_shape = (self.batch, self.kv_heads, self.seq, self.dim)
         return [(q, "q", self.torch_dtype, self._shape()), (k, "k", self.torch_dtype, kv_shape),
@@ -140,48 +160,55 @@ class RingAttention:
 
     def block_forward(self, step, q, k, v, o_part=None, lse_part=None, stream=None):
         specs = self._qkv_specs(q, k, v)
+        # slot-major partials: the slot of this step; row-major (row_partials): the whole buffers, for every step
+        o_shape, l_shape = self.parts_shapes() if self.row_partials else (self._shape(), self._shape()[:3])
         if o_part is not None:
-            specs.append((o_part, "o_part", self.part_dtype, self._shape()))
+            specs.append((o_part, "o_part", self.part_dtype, o_shape))
         if lse_part is not None:
-            specs.append((lse_part, "lse_part", torch.float32, self._shape()[:3]))
+            specs.append((lse_part, "lse_part", torch.float32, l_shape))
         _check_tensors(*specs)
         if o_part is None:
-            o_part = torch.zeros(self._shape(), dtype=self.part_dtype, device=q.device)
+            o_part = torch.zeros(o_shape, dtype=self.part_dtype, device=q.device)
         if lse_part is None:
-            lse_part = torch.full(self._shape()[:3], float("-inf"), dtype=torch.float32, device=q.device)
+            lse_part = torch.full(l_shape, float("-inf"), dtype=torch.float32, device=q.device)
         check(self.lib.ringattn_block_fwd(self.handle, int(step), _ptr(q), _ptr(k), _ptr(v), _ptr(o_part),
                                           _ptr(lse_part), _stream_ptr(stream)), "ringattn_block_fwd")
         return o_part, lse_part
 
     def rank_step_forward(self, rank, step, q, k_chunk, v_chunk, o_part=None, lse_part=None, stream=None):
         """One ring step of one rank on rank-local tensors (q: the rank's rows; k_chunk, v_chunk: the
-        chunk of rank (rank + step) % npes).  Returns the rank-local partial (O, LSE)."""
+        chunk of rank (rank + step) % npes).  Returns the rank-local partial (O, LSE); on a plan with row_partials
+        o_part and lse_part are the rank's whole [B, H, rows, npes, d] / [B, H, rows, npes] buffers at every step."""
         if not (0 <= rank < self.npes and 0 <= step < self.npes):
             raise ValueError("rank and step must be in [0, npes)")
         rows, kv_rows = self.seqlen[rank], self.seqlen[(rank + step) % self.npes]
+        o_shape, l_shape = (self.batch, self.heads, rows, self.dim), (self.batch, self.heads, rows)
+        if self.row_partials:
+            o_shape, l_shape = self.rank_parts_shapes(rank)
         specs = [(q, "q", self.torch_dtype, (self.batch, self.heads, rows, self.dim)),
                  (k_chunk, "k_chunk", self.torch_dtype, (self.batch, self.kv_heads, kv_rows, self.dim)),
                  (v_chunk, "v_chunk", self.torch_dtype, (self.batch, self.kv_heads, kv_rows, self.dim))]
         if o_part is not None:
-            specs.append((o_part, "o_part", self.part_dtype, (self.batch, self.heads, rows, self.dim)))
+            specs.append((o_part, "o_part", self.part_dtype, o_shape))
         if lse_part is not None:
-            specs.append((lse_part, "lse_part", torch.float32, (self.batch, self.heads, rows)))
+            specs.append((lse_part, "lse_part", torch.float32, l_shape))
         _check_tensors(*specs)
         if o_part is None:
-            o_part = torch.zeros((self.batch, self.heads, rows, self.dim), dtype=self.part_dtype, device=q.device)
+            o_part = torch.zeros(o_shape, dtype=self.part_dtype, device=q.device)
         if lse_part is None:
-            lse_part = torch.full((self.batch, self.heads, rows), float("-inf"), dtype=torch.float32, device=q.device)
+            lse_part = torch.full(l_shape, float("-inf"), dtype=torch.float32, device=q.device)
         check(self.lib.ringattn_rank_step_fwd(self.handle, int(rank), int(step), _ptr(q), _ptr(k_chunk), _ptr(v_chunk),
                                               _ptr(o_part), _ptr(lse_part), _stream_ptr(stream)), "ringattn_rank_step_fwd")
         return o_part, lse_part
 
     def rank_merge(self, rank, o_parts, lse_parts, out=None, lse=None, stream=None):
-        """Merge of one rank's per-step partials [npes, B, H, rows, d] / [npes, B, H, rows]."""
+        """Merge of one rank's per-step partials [npes, B, H, rows, d] / [npes, B, H, rows]
+        ([B, H, rows, npes, d] / [B, H, rows, npes] on a plan with row_partials)."""
         if not 0 <= rank < self.npes:
             raise ValueError("rank must be in [0, npes)")
         rows = self.seqlen[rank]
-        _check_tensors((o_parts, "o_parts", self.part_dtype, (self.npes, self.batch, self.heads, rows, self.dim)),
-                       (lse_parts, "lse_parts", torch.float32, (self.npes, self.batch, self.heads, rows)))
+        o_shape, l_shape = self.rank_parts_shapes(rank)
+        _check_tensors((o_parts, "o_parts", self.part_dtype, o_shape), (lse_parts, "lse_parts", torch.float32, l_shape))
         if out is None:
             out = torch.empty((self.batch, self.heads, rows, self.dim), dtype=self.torch_dtype, device=o_parts.device)
         if lse is None:
@@ -226,9 +253,10 @@ class RingAttention:
         return [(st[i], ln[i], act[i]) for i in range(n.value)]
 
     def merge_ring(self, o_parts, lse_parts, out=None, lse=None, stream=None):
-        """Ring-aware merge of caller-held per-step partials [npes, B, H, S, d] / [npes, B, H, S]."""
-        _check_tensors((o_parts, "o_parts", self.part_dtype, (self.npes,) + self._shape()),
-                       (lse_parts, "lse_parts", torch.float32, (self.npes,) + self._shape()[:3]))
+        """Ring-aware merge of caller-held per-step partials [npes, B, H, S, d] / [npes, B, H, S]
+        ([B, H, S, npes, d] / [B, H, S, npes] on a plan with row_partials)."""
+        o_shape, l_shape = self.parts_shapes()
+        _check_tensors((o_parts, "o_parts", self.part_dtype, o_shape), (lse_parts, "lse_parts", torch.float32, l_shape))
         if out is None:
             out = torch.empty(self._shape(), dtype=self.torch_dtype, device=o_parts.device)
         if lse is None:

@@ -92,6 +92,7 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 inline bool half_partials(const ringattn_params& p) { return (p.flags & RINGATTN_FLAG_HALF_PARTIALS) != 0; }
 inline bool step_partials(const ringattn_params& p) { return (p.flags & RINGATTN_FLAG_STEP_PARTIALS) != 0; }
+inline bool row_partials(const ringattn_params& p) { return (p.flags & RINGATTN_FLAG_ROW_PARTIALS) != 0; }
 
 inline ringattn::WorkItem make_item(int q_start, int q_len, int kv_start, int kv_len, int diag_off, int slot) {
   ringattn::WorkItem w;
@@ -284,7 +285,8 @@ inline int q_tiles_of(int len) { return (len + ringattn::kWalkM - 1) / ringattn:
 // partial block lives.  A masked (diagonal) item runs last and the q tiles go busiest first.
 template <class BaseFn>
 void push_segment(ringattn_plan* pl, TableSlice& slice, int q_start, int q_len,
-                  const std::vector<ringattn::WorkItem>& items, int kv_shift, BaseFn part_base, int part_bh_stride) {
+                  const std::vector<ringattn::WorkItem>& items, int kv_shift, BaseFn part_base, int part_bh_stride,
+                  int part_row_mul = 0) {
   ringattn::Segment sg;
   std::memset(&sg, 0, sizeof(sg));
   sg.q_start = q_start;
@@ -302,6 +304,7 @@ void push_segment(ringattn_plan* pl, TableSlice& slice, int q_start, int q_len,
     it.part_bh_stride = part_bh_stride;
     it.part_base = part_base((int)i);
     it.slot = w.slot;
+    it.part_row_mul = part_row_mul;
     if (w.diag_off >= 0) {
       sg.last_item = (int)i;
       sg.reverse_tiles = 1;
@@ -369,7 +372,8 @@ void build_schedule(ringattn_plan* pl) {
       for (const auto& w : one) {
         pl->h_items.push_back(w);
         const std::vector<ringattn::WorkItem> v1{w};
-        push_segment(pl, sl, w.q_start, w.q_len, v1, 0, [&](int) { return (int64_t)w.q_start; }, (int)d.S);
+        push_segment(pl, sl, w.q_start, w.q_len, v1, 0, [&](int) { return (int64_t)w.q_start; }, (int)d.S,
+                     row_partials(pl->p) ? P : 0);
       }
     }
     pl->step.push_back(sl);
@@ -386,7 +390,8 @@ void build_schedule(ringattn_plan* pl) {
       const int q0 = d.start[r], rows = d.start[r + 1] - q0, k0 = d.start[(r + s) % P];
       for (const auto& w : one) {
         const std::vector<ringattn::WorkItem> v1{w};
-        push_segment(pl, sl, w.q_start - q0, w.q_len, v1, k0, [&](int) { return (int64_t)(w.q_start - q0); }, rows);
+        push_segment(pl, sl, w.q_start - q0, w.q_len, v1, k0, [&](int) { return (int64_t)(w.q_start - q0); }, rows,
+                     row_partials(pl->p) ? P : 0);
       }
       pl->local.push_back(sl);
     }
@@ -641,6 +646,7 @@ int launch_regions(const ringattn_plan* pl, int first, int count, int max_len, i
   m.S = rows_per_head;
   m.part_stride_rows = part_stride_rows;
   m.half_partials = half_partials(pl->p) ? 1 : 0;
+  m.row_mul = row_partials(pl->p) ? pl->p.npes : 0;
   RA_HIP(ringattn::launch_merge(m, pl->p.dtype, pl->p.dim, stream));
   return RINGATTN_OK;
 }

@@ -36,8 +36,9 @@ struct SegItem {
   int diag_off;         // as in WorkItem, relative to the first row of the segment
   int part_bh_stride;   // rows between consecutive heads in this item's partial block
   int64_t part_base;    // row (in the partial buffers) of the segment's first row of head 0
-  int slot;             // ring step, for inspection only
-  int pad;
+  int slot;             // ring step: the entry of a row's run with row-major partials, else for inspection only
+  int part_row_mul;     // 0: the partial of row r lives at row r of the buffers; n > 0: at entry n r + slot (a row's
+                        // steps next to each other, n of them)
 };
 static_assert(sizeof(SegItem) == 32, "SegItem is read as two 16-byte scalar loads");
 
@@ -107,6 +108,7 @@ struct MergeArgs {
   int S;                  // rows per head
   int64_t part_stride_rows;  // rows between consecutive slots (>= heads * S)
   int half_partials;
+  int row_mul;            // 0: slot-major partials as above; n > 0: [heads * S, n, D] / [heads * S, n], a row's slots adjacent
 };
 
 // Up to kMaxParts table entries passed BY VALUE to a small kernel that writes them to device

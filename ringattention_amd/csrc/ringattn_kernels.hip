@@ -95,7 +95,8 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
   const int64_t idx = (int64_t)blockIdx.x * ROWS + threadIdx.x / TPR;  // over heads x reg.len
   if (idx >= (int64_t)a.heads * reg.len) return;
   const int64_t row = (idx / reg.len) * a.S + reg.start + idx % reg.len;
-  SlotParts parts{reg.active, row, a.part_stride_rows};
+  // slot-major partials: slot s of a row lies part_stride_rows rows further on; row-major: at entry row_mul row + s
+  SlotParts parts{reg.active, a.row_mul > 0 ? row * a.row_mul : row, a.row_mul > 0 ? (int64_t)1 : a.part_stride_rows};
   merge_row<DT, D, HP>(parts, a.o_parts, a.lse_parts, a.out, a.lse, row, threadIdx.x % TPR);
 }
 

@@ -48,6 +48,7 @@ uint64_t g_clock = 0;
 std::shared_ptr<Entry> plan_for(const PlanKey& key, const ringattn_params& p) {
   std::vector<std::shared_ptr<Entry>> evicted;
   std::shared_ptr<Entry> e;
+  int create_rc = RINGATTN_OK;
   {
     std::lock_guard<std::mutex> lk(g_mu);
     auto it = g_plans.find(key);
@@ -65,11 +66,17 @@ std::shared_ptr<Entry> plan_for(const PlanKey& key, const ringattn_params& p) {
     }
     e = std::make_shared<Entry>();
     const int rc = ringattn_plan_create(&p, nullptr, 0, &e->plan);
-    TORCH_CHECK(rc == RINGATTN_OK, "ringattn_plan_create: ", ringattn_strerror(rc));
-    e->last_use = ++g_clock;
-    g_plans.emplace(key, e);
+    if (rc == RINGATTN_OK) {
+      e->last_use = ++g_clock;
+      g_plans.emplace(key, e);
+    } else {
+      e.reset();
+    }
+    create_rc = rc;
   }
+  // outside the lock, and whether or not the new plan came to be: the evicted plans go back to the device
   for (auto& v : evicted) (void)ringattn_plan_destroy(v->plan);
+  TORCH_CHECK(create_rc == RINGATTN_OK, "ringattn_plan_create: ", ringattn_strerror(create_rc));
   return e;
 }
 

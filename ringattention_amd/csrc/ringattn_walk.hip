@@ -354,7 +354,8 @@ __global__ __launch_bounds__(512, 1) void ring_walk_kernel(const BlockArgs a) {
     const float inv = (l > 0.f) ? 1.f / l : 0.f;
     const int row_l = qt * BM + 32 * wave + n;
     if (row_l >= q_len) return;  // a row beyond the query range
-    const int64_t prow = w->part_base + (int64_t)bh * w->part_bh_stride + row_l;
+    int64_t prow = w->part_base + (int64_t)bh * w->part_bh_stride + row_l;
+    if (w->part_row_mul > 0) prow = prow * w->part_row_mul + w->slot;  // a row's steps next to each other
     const int64_t opos = prow * D;
 #pragma unroll
     for (int db = 0; db < DB; ++db)

@@ -502,6 +502,35 @@ def test_block_step_and_merge_separately(oracle, causal):
     check_rows(oracle, w, q, k, v, out, lse, rows)
 
 
+@pytest.mark.parametrize("causal,half,d", [(False, False, 128), (True, False, 128), (True, True, 64), (False, True, 128)])
+def test_row_major_partials_give_the_bits_of_slot_major_ones(causal, half, d):
+    """RINGATTN_FLAG_ROW_PARTIALS only changes where a partial is kept ([rows, steps, d]: a row's steps next to each
+    other): the steps, run one by one, write the numbers of the slot-major layout to their new places, and the ring
+    merge gives the same bits."""
+    w = Workload("rowparts", 2, 2, d, 4, 320, "bf16" if d == 128 else "fp16", 47, causal)
+    q, k, v = api.make_qkv_bits(w)
+    qd, kd, vd = (to_dev(x, w.dtype) for x in (q, k, v))
+    results = []
+    for row_major in (False, True):
+        plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, half_partials=half,
+                                 row_partials=row_major)
+        o_shape, l_shape = plan.parts_shapes()
+        o_parts = torch.zeros(o_shape, dtype=plan.part_dtype, device="cuda")
+        l_parts = torch.full(l_shape, float("-inf"), dtype=torch.float32, device="cuda")
+        for s in range(w.npes):
+            if row_major:
+                plan.block_forward(s, qd, kd, vd, o_parts, l_parts)
+            else:
+                plan.block_forward(s, qd, kd, vd, o_parts[s], l_parts[s])
+        out, lse = plan.merge_ring(o_parts, l_parts)
+        torch.cuda.synchronize()
+        plan.close()
+        results.append((o_parts, l_parts, out, lse))
+    (o_s, l_s, out_s, lse_s), (o_r, l_r, out_r, lse_r) = results
+    assert torch.equal(o_s.permute(1, 2, 3, 0, 4), o_r) and torch.equal(l_s.permute(1, 2, 3, 0), l_r)
+    assert torch.equal(out_s.view(torch.int16), out_r.view(torch.int16)) and torch.equal(lse_s, lse_r)
+
+
 def test_merge_identity_and_random_parts(oracle):
     rng = np.random.default_rng(3)
     n, rows, d = 7, 1000, 64
@@ -742,4 +771,21 @@ def test_rank_local_ring_equals_the_all_rank_forward(seqlen, causal, layout, d, 
         o_r, l_r = plan.rank_merge(r, o_parts, l_parts)
         torch.cuda.synchronize()
         assert torch.equal(o_r, out[:, :, rows]) and torch.equal(l_r, lse[:, :, rows]), f"rank {r}"
+    plan.close()
+    # the same ring with a row's steps next to each other in the rank's partials (RINGATTN_FLAG_ROW_PARTIALS)
+    plan = api.RingAttention(P, list(seqlen), d, B, H, dtype, causal, kv_heads=hkv, layout=layout, half_partials=half,
+                             row_partials=True)
+    for r in range(P):
+        rows = slice(start[r], start[r + 1])
+        q_r = qd[:, :, rows].contiguous()
+        o_shape, l_shape = plan.rank_parts_shapes(r)
+        o_parts = torch.zeros(o_shape, dtype=plan.part_dtype, device="cuda")
+        l_parts = torch.full(l_shape, float("-inf"), dtype=torch.float32, device="cuda")
+        for s in range(P):
+            j = (r + s) % P
+            plan.rank_step_forward(r, s, q_r, kd[:, :, start[j]:start[j + 1]].contiguous(),
+                                   vd[:, :, start[j]:start[j + 1]].contiguous(), o_parts, l_parts)
+        o_r, l_r = plan.rank_merge(r, o_parts, l_parts)
+        torch.cuda.synchronize()
+        assert torch.equal(o_r, out[:, :, rows]) and torch.equal(l_r, lse[:, :, rows]), f"rank {r}, row-major partials"
     plan.close()
