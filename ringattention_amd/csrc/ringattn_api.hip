@@ -209,12 +209,17 @@ struct TableSlice {
   bool wide = false;    // every KV range of the slice suits ring_walk64_kernel
 };
 
-// ring_walk64_kernel walks whole 32-key tiles and steps its load streams four tiles at a time: a KV range must
-// be a multiple of 32 keys and hold at least 128.
+// ring_walk64_kernel walks whole 32-key tiles, and past the end of its sequence its load streams go round the first
+// four tiles of a head: a KV range must be a multiple of 32 keys and hold at least 128.
 static bool walk64_takes(const ringattn::SegItem& it) { return it.kv_len % 32 == 0 && it.kv_len >= 128; }
 // RINGATTN_WIDE=0 in the environment keeps every forward on ring_walk_kernel (for comparisons)
 static bool walk64_enabled() {
   const char* e = std::getenv("RINGATTN_WIDE");
+  return !(e && e[0] == '0');
+}
+// RINGATTN_WIDE_PARTIALS=0 keeps the launches that emit per-step partials on ring_walk_kernel
+static bool walk64_partials_enabled() {
+  const char* e = std::getenv("RINGATTN_WIDE_PARTIALS");
   return !(e && e[0] == '0');
 }
 
@@ -313,6 +318,9 @@ void push_segment(ringattn_plan* pl, TableSlice& slice, int q_start, int q_len,
   }
   if (sg.item_count == 1) sg.last_item = -1;
   pl->h_segs.push_back(sg);
+  bool wide = true;
+  for (size_t i = 0; i < items.size(); ++i) wide = wide && walk64_takes(pl->h_segitems[(size_t)sg.item_begin + i]);
+  slice.wide = slice.seg_count == 0 ? wide : (slice.wide && wide);
   ++slice.seg_count;
   slice.q_tiles_max = std::max(slice.q_tiles_max, q_tiles_of(q_len));
 }
@@ -342,8 +350,6 @@ void build_schedule(ringattn_plan* pl) {
     }
   }
   pl->fwd_items = (int)pl->h_items.size();
-  pl->fwd.wide = true;
-  for (const auto& it : pl->h_segitems) pl->fwd.wide = pl->fwd.wide && walk64_takes(it);
   // Workgroup order of the forward.  Heads are dealt to the 8 XCDs round-robin; an XCD runs
   // the segments of one head after the other (busiest first within a head), so the ranks of
   // a head, which read the same K and V, follow each other through that XCD's L2.  Only when
@@ -440,10 +446,11 @@ int ensure_tables(ringattn_plan* pl) {
   return RINGATTN_OK;
 }
 
-// ring_walk64_kernel runs the carried-state launch of a slice when every KV range suits it, d = 128, and a head is
-// long enough for the loads it issues past the last chunk (whole tiles from the start of the head, never read back)
-bool slice_takes_walk64(const ringattn_plan* pl, const TableSlice& sl) {
-  return sl.wide && pl->p.dim == 128 && pl->d.S >= 512 && walk64_enabled();
+// ring_walk64_kernel runs the launch of a slice when every KV range suits it and d = 128.  The launches that emit
+// partials go by the forward's ranges, so that the forward and the steps run one by one keep giving the same bits.
+bool slice_takes_walk64(const ringattn_plan* pl, const TableSlice& sl, int mode) {
+  if (mode != ringattn::kBlockCarryState && !(walk64_partials_enabled() && pl->fwd.wide)) return false;
+  return sl.wide && pl->p.dim == 128 && walk64_enabled();
 }
 
 // A block launch over a slice of the tables.
@@ -453,7 +460,7 @@ int launch_slice(const ringattn_plan* pl, const TableSlice& sl, ringattn::BlockA
   a.items = pl->d_segitems;
   a.n_segs = sl.seg_count;
   a.q_tiles_max = sl.q_tiles_max;
-  if (a.mode == ringattn::kBlockCarryState && slice_takes_walk64(pl, sl))
+  if (slice_takes_walk64(pl, sl, a.mode))
     RA_HIP(ringattn::launch_walk64(a, pl->p.dtype, stream));
   else
     RA_HIP(ringattn::launch_walk(a, pl->p.dtype, pl->p.dim, stream));
@@ -588,7 +595,7 @@ int run_rank_call(const RankCall& rc, void* scratch, const void* q, const void* 
   a.q_tiles_max = q_tiles_of(c);
   a.bh_stride = (int64_t)c * dim;  // q and out hold this rank's rows only; k and v the whole sequence
   a.S = c;
-  bool wide = dim == 128 && rc.d.S >= 512 && walk64_enabled();
+  bool wide = dim == 128 && walk64_enabled();
   for (int i = 0; i < n_parts; ++i) wide = wide && walk64_takes(rc.pack.items[i]);
   if (wide) RA_HIP(ringattn::launch_walk64(a, rc.p.dtype, stream));
   else RA_HIP(ringattn::launch_walk(a, rc.p.dtype, dim, stream));
@@ -873,7 +880,8 @@ int ringattn_plan_launch_times(ringattn_plan* plan, float* ms, int capacity, int
 
 const char* ringattn_plan_forward_kernel(const ringattn_plan* plan) {
   if (!plan_ok(plan)) return nullptr;
-  return (!step_partials(plan->p) && slice_takes_walk64(plan, plan->fwd)) ? "ring_walk64_kernel" : "ring_walk_kernel";
+  const int mode = step_partials(plan->p) ? ringattn::kBlockPartialsMerged : ringattn::kBlockCarryState;
+  return slice_takes_walk64(plan, plan->fwd, mode) ? "ring_walk64_kernel" : "ring_walk_kernel";
 }
 
 int ringattn_plan_merge_regions(const ringattn_plan* plan, int* start, int* len, uint64_t* active, int capacity, int* n_out) {

@@ -18,15 +18,18 @@
 //       One wave per SIMD has nobody to wait behind, so nothing may be waited for: the K and V rings are eight
 //       tiles deep (128 KB of LDS) and a tile is loaded four or more iterations before the barrier that hands it
 //       over (s_waitcnt vmcnt(12): the loads of the last three iterations stay in flight).
-//       Shapes it takes: every KV range a multiple of 32 keys and at least 128, at least 512 rows per head (the
-//       host checks); anything else runs ring_walk_kernel.
+//       Shapes it takes: every KV range a multiple of 32 keys and at least 128 (the host checks); anything else
+//       runs ring_walk_kernel.
 #include "ringattn_device.h"
 
 #include <type_traits>
 
 namespace ringattn {
 
-template <int DT>
+// KEEP: max / sum / acc-O run through all chunks of the q tile and the rows' result is written once (kBlockCarryState).
+// Otherwise the chunks are walked one by one, each as a sequence of its own -- prologue, loop, drain --, and each
+// ends in its normalised partial (O, LSE) (kBlockPartials, kBlockPartialsMerged; HP: partial O as fp16).
+template <int DT, bool KEEP, bool HP>
 __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) {
   using E = Elem<DT>;
   constexpr int D = 128;
@@ -42,7 +45,7 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
   constexpr float kLazyLog2 = 8.f;
   static_assert(BM == 64 * WAVES, "two 32-row blocks per wave");
   constexpr int kListAt = 2 * NBUF * TILE;  // behind the rings: the chunks of this q tile in walking order, (byte offset, tiles) each
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[kListAt + 8 * (kMaxParts + 2)];
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[kListAt + 8 * (kMaxParts + 4)];
 
   const unsigned smem_base = lds_offset(smem);
   const int tid = threadIdx.x, lane = tid & 63;
@@ -53,11 +56,11 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
   int bh, qt;
   if (!decode_job<BM>(a, seg, bh, qt)) return;
   const int q_start = seg.q_start, q_len = seg.q_len;
-  const int n_items = seg.item_count;
+  const int all_items = seg.item_count;
   // items in run order: table order, except that item `last_item` (the diagonal one) is moved to the end
-  auto item_at = [&](int i) -> const SegItem* {
+  auto item_in_order = [&](int i) -> const SegItem* {
     int idx = i;
-    if (seg.last_item >= 0) idx = (i == n_items - 1) ? seg.last_item : (i >= seg.last_item ? i + 1 : i);
+    if (seg.last_item >= 0) idx = (i == all_items - 1) ? seg.last_item : (i >= seg.last_item ? i + 1 : i);
     return a.items + seg.item_begin + idx;
   };
   const int64_t head_off = (int64_t)bh * a.bh_stride;
@@ -98,7 +101,11 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
     }
   }
 
-  // ---- the flattened tile sequence of this q tile: item i contributes tiles_of(i) tiles
+  // ---- a pass walks n_items chunks from item `first` on as one sequence: all of them (KEEP), or one
+  const int n_items = KEEP ? all_items : 1;
+  for (int first = 0; first < all_items; first += n_items) {
+  auto item_at = [&](int i) -> const SegItem* { return item_in_order(first + i); };
+  // ---- the flattened tile sequence of the pass: item i contributes tiles_of(i) tiles
   const int diag_item = (n_items > 0 && item_at(n_items - 1)->diag_off >= 0) ? n_items - 1 : -1;
   auto tiles_of = [&](const SegItem* w) {
     const int kv_tiles = w->kv_len / BN;
@@ -118,8 +125,9 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
   }
 
   // ---- load streams: K is loaded seven to eight tiles ahead of its product, V four to five.  A stream is a byte
-  // offset from the head's first row; past the last chunk it wraps to the start of the head (whole tiles of valid
-  // memory that nobody reads from LDS), so that every iteration issues the same number of loads.
+  // offset from the head's first row; past the last chunk it goes round the first four tiles of the head (valid
+  // memory: some KV range of 128 keys lies in every head; nobody reads these tiles from LDS), so that every
+  // iteration issues the same number of loads.  At most nine tiles are loaded past the end: three such rounds.
   struct Stream {
     unsigned off;  // the next tile to load
     int left;      // tiles left in its chunk, that one included
@@ -132,7 +140,7 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
       cnt = tiles_of(w);
     } else {
       off = 0;
-      cnt = 0x40000000;
+      cnt = 4;
     }
   };
   auto step = [&](Stream& s) {
@@ -333,9 +341,10 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
 
   // ---- prologue: K(0) .. K(6) and V(0) .. V(4) next to the Q loads; the scores of tile 0.  V ring slot 7 -- "tile
   // -1", which the first iteration multiplies with all-zero probabilities -- is cleared.
+  if (first > 0) __syncthreads();  // every wave is done with the rings and the chunk list of the pass before
   for (int t = 0; t < 7; ++t) issue_k(t);
   for (int t = 0; t < 5; ++t) issue_v(t);
-  if (tid < n_items + 2) {  // the chunk list the hand-scheduled loop steps its load streams through
+  if (tid < n_items + 4) {  // the chunk list the hand-scheduled loop steps its load streams through
     unsigned o;
     int c;
     chunk_of(tid, o, c);
@@ -396,28 +405,65 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   if (pend) settle(false);
 
-  // ---- the rows' result: the reference's epilogue (csrc/ring_attention.cu:621-664), O = acc / l in the storage
-  // type, plus the LSE
+  if (KEEP) {
+    // ---- the rows' result: the reference's epilogue (csrc/ring_attention.cu:621-664), O = acc / l in the storage
+    // type, plus the LSE
 #pragma unroll
-  for (int b = 0; b < 2; ++b) {
-    const float l = cross_half_sum((ls[b][0] + ls[b][1]) + (ls[b][2] + ls[b][3]));
-    const float inv = (l > 0.f) ? 1.f / l : 0.f;
-    const int row_l = qt * BM + 64 * wave + 32 * b + n;
-    if (row_l < q_len) {  // not a row beyond the query range
-      const int64_t row = (int64_t)bh * a.S + q_start + row_l;
-      typename E::type* orow = (typename E::type*)a.out + row * D;
+    for (int b = 0; b < 2; ++b) {
+      const float l = cross_half_sum((ls[b][0] + ls[b][1]) + (ls[b][2] + ls[b][3]));
+      const float inv = (l > 0.f) ? 1.f / l : 0.f;
+      const int row_l = qt * BM + 64 * wave + 32 * b + n;
+      if (row_l < q_len) {  // not a row beyond the query range
+        const int64_t row = (int64_t)bh * a.S + q_start + row_l;
+        typename E::type* orow = (typename E::type*)a.out + row * D;
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          typename E::vec4 val;
+          for (int q4 = 0; q4 < 4; ++q4) {
+            typename E::vec4 val;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) val[e] = (typename E::type)(oacc[b][db][4 * q4 + e] * inv);
-          *(typename E::vec4*)(orow + 32 * db + 8 * q4 + 4 * h) = val;
-        }
-      if (h == 0 && a.lse) a.lse[row] = (l > 0.f) ? (ms[b] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
+            for (int e = 0; e < 4; ++e) val[e] = (typename E::type)(oacc[b][db][4 * q4 + e] * inv);
+            *(typename E::vec4*)(orow + 32 * db + 8 * q4 + 4 * h) = val;
+          }
+        if (h == 0 && a.lse) a.lse[row] = (l > 0.f) ? (ms[b] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
+      }
+    }
+  } else {
+    // ---- the chunk's partial (csrc/ring_attention.cu:621-633): normalised O and LSE at the rows of the queries
+    const SegItem* w = item_at(0);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const float l = cross_half_sum((ls[b][0] + ls[b][1]) + (ls[b][2] + ls[b][3]));
+      const float inv = (l > 0.f) ? 1.f / l : 0.f;
+      const int row_l = qt * BM + 64 * wave + 32 * b + n;
+      if (row_l < q_len) {
+        int64_t prow = w->part_base + (int64_t)bh * w->part_bh_stride + row_l;
+        if (w->part_row_mul > 0) prow = prow * w->part_row_mul + w->slot;  // a row's steps next to each other
+        const int64_t opos = prow * D;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            f32x4 val;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) val[e] = oacc[b][db][4 * q4 + e] * inv;
+            if (HP) {  // fp16 partials: |O_part| <= max |V|, the caller vouches that this fits
+              f16x4 hv;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) hv[e] = (_Float16)val[e];
+              *(f16x4*)((_Float16*)a.o_part + opos + 32 * db + 8 * q4 + 4 * h) = hv;
+            } else {
+              *(f32x4*)((float*)a.o_part + opos + 32 * db + 8 * q4 + 4 * h) = val;
+            }
+          }
+        if (h == 0) a.lse_part[prow] = (l > 0.f) ? (ms[b] + __builtin_amdgcn_logf(l)) * 0.6931471805599453f : -INFINITY;
+      }
     }
   }
+  }  // passes
+  if (!KEEP && a.mode == kBlockPartialsMerged)  // this workgroup's rows over the partials it has just written
+    merge_job_rows<DT, D, HP, BM, 64 * WAVES>(a.o_part, a.lse_part, a.out, a.lse, a.items, seg, bh, qt, a.S,
+                                              (lds_float*)(__attribute__((address_space(3))) void*)smem);
 }
 
 hipError_t launch_walk64(const BlockArgs& a, int dtype, hipStream_t stream) {
@@ -425,11 +471,19 @@ hipError_t launch_walk64(const BlockArgs& a, int dtype, hipStream_t stream) {
   const int q_tiles = a.q_tiles_max;
   const int64_t groups = (int64_t)a.n_segs * a.BH;
   const int64_t blocks = (a.groups ? (int64_t)a.groups_per_xcd : (groups + 7) / 8) * 8 * q_tiles;
-  if (q_tiles <= 0 || blocks > INT32_MAX || a.mode != kBlockCarryState) return hipErrorInvalidValue;
+  if (q_tiles <= 0 || blocks > INT32_MAX) return hipErrorInvalidValue;
+  if (a.mode != kBlockCarryState && a.mode != kBlockPartials && a.mode != kBlockPartialsMerged) return hipErrorInvalidValue;
   const unsigned grid = (unsigned)blocks;
-  if (dtype == 0) ring_walk64_kernel<0><<<grid, 256, 0, stream>>>(a);
-  else if (dtype == 1) ring_walk64_kernel<1><<<grid, 256, 0, stream>>>(a);
+#define RA_LAUNCH_WALK64(DT_)                                                                       \
+  do {                                                                                             \
+    if (a.mode == kBlockCarryState) ring_walk64_kernel<DT_, true, false><<<grid, 256, 0, stream>>>(a);  \
+    else if (a.half_partials) ring_walk64_kernel<DT_, false, true><<<grid, 256, 0, stream>>>(a);        \
+    else ring_walk64_kernel<DT_, false, false><<<grid, 256, 0, stream>>>(a);                            \
+  } while (0)
+  if (dtype == 0) RA_LAUNCH_WALK64(0);
+  else if (dtype == 1) RA_LAUNCH_WALK64(1);
   else return hipErrorInvalidValue;
+#undef RA_LAUNCH_WALK64
   return hipGetLastError();
 }
 

@@ -55,6 +55,8 @@ def test_reference_moves_inside_the_hand_scheduled_loop(oracle, w, slope, period
     Workload("w_c1", 1, 2, 128, 1, 2048, "bf16", 53, True),        # one chunk, all of it diagonal
     Workload("w_min", 1, 2, 128, 4, 128, "bf16", 54, True),        # the shortest chunks the kernel takes (4 tiles)
     Workload("w_big", 1, 2, 128, 2, 1024, "fp16", 55, False, sigma_qk=3.0),
+    Workload("w_tiny", 1, 2, 128, 1, 128, "bf16", 56, True),       # half a q tile: two waves own no row at all
+    Workload("w_short", 2, 1, 128, 2, 160, "fp16", 57, False),     # heads shorter than what the load streams run ahead
 ], ids=lambda w: w.name)
 def test_both_kernels_agree(oracle, w, monkeypatch):
     """The same forward with and without RINGATTN_WIDE=0 (which keeps it on ring_walk_kernel): both against the oracle,
@@ -102,3 +104,49 @@ def test_wide_kernel_with_grouped_heads_and_unequal_ranks(oracle):
     finally:
         plan.close()
     check_rows(oracle, wu, q, k, v, out, lse, np.arange(wu.rows))
+
+
+@pytest.mark.parametrize("w,half", [
+    (Workload("p_nc", 1, 3, 128, 4, 512, "bf16", 71, False), False),
+    (Workload("p_c", 2, 2, 128, 4, 384, "fp16", 72, True), False),
+    (Workload("p_c_half", 1, 2, 128, 8, 256, "fp16", 73, True), True),
+    (Workload("p_min", 1, 2, 128, 3, 128, "bf16", 74, True), False),   # four-tile chunks, a q tile and a half per head
+    (Workload("p_rise", 1, 2, 128, 2, 1024, "bf16", 75, True), False),
+], ids=lambda x: x.name if isinstance(x, Workload) else None)
+def test_chunk_by_chunk_walk_with_partials(oracle, w, half, monkeypatch):
+    """The forward that keeps the ring steps apart (a partial (O, LSE) per chunk, merged at the end) on
+    ring_walk64_kernel, which then walks every chunk as a sequence of its own: against the oracle, against the same
+    forward on ring_walk_kernel (RINGATTN_WIDE_PARTIALS=0), and, bit for bit, against the steps launched one by one
+    with a separate merge."""
+    q, k, v = rising_logits(w, 0.25) if w.name == "p_rise" else api.make_qkv_bits(w)
+    qd, kd, vd = (api.bits_to_tensor(x, w.dtype) for x in (q, k, v))
+
+    def run():
+        plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, step_partials=True,
+                                 half_partials=half)
+        try:
+            out, lse = plan.forward(qd, kd, vd)
+            o_shape, l_shape = plan.parts_shapes()
+            o_parts = torch.zeros(o_shape, dtype=plan.part_dtype, device="cuda")
+            l_parts = torch.full(l_shape, float("-inf"), dtype=torch.float32, device="cuda")
+            for s in range(w.npes):
+                plan.block_forward(s, qd, kd, vd, o_parts[s], l_parts[s])
+            out_m, lse_m = plan.merge_ring(o_parts, l_parts)
+            torch.cuda.synchronize()
+        finally:
+            plan.close()
+        assert torch.equal(out.view(torch.int16), out_m.view(torch.int16)) and torch.equal(lse, lse_m)
+        return out, lse
+
+    monkeypatch.delenv("RINGATTN_WIDE", raising=False)
+    monkeypatch.delenv("RINGATTN_WIDE_PARTIALS", raising=False)
+    out_w, lse_w = run()
+    check_rows(oracle, w, q, k, v, out_w, lse_w, np.arange(w.rows))
+    monkeypatch.setenv("RINGATTN_WIDE_PARTIALS", "0")
+    out_b, lse_b = run()
+    a, b = out_w.double().cpu().numpy().reshape(-1, w.dim), out_b.double().cpu().numpy().reshape(-1, w.dim)
+    big = np.maximum(np.abs(a), np.abs(b)).max(axis=1, keepdims=True)
+    mant = 10 if w.dtype == "fp16" else 7
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(big, 2.0 ** -14))) - mant)
+    assert (np.abs(a - b) <= (3 if half else 2) * ulp).all()
+    assert np.abs(lse_w.double().cpu().numpy() - lse_b.double().cpu().numpy()).max() <= 1e-4
