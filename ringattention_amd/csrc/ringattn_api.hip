@@ -207,6 +207,7 @@ struct TableSlice {
   int seg_begin = 0, seg_count = 0;
   int q_tiles_max = 0;  // kWalkM-row tiles of the longest segment
   bool wide = false;    // every KV range of the slice suits ring_walk64_kernel
+  int min_kv = 0;       // the shortest KV range of the slice
 };
 
 // ring_walk64_kernel walks whole 32-key tiles, and past the end of its sequence its load streams go round the first
@@ -217,10 +218,11 @@ static bool walk64_enabled() {
   const char* e = std::getenv("RINGATTN_WIDE");
   return !(e && e[0] == '0');
 }
-// RINGATTN_WIDE_PARTIALS=0 keeps the launches that emit per-step partials on ring_walk_kernel
-static bool walk64_partials_enabled() {
+// RINGATTN_WIDE_PARTIALS in the environment: 0 keeps the launches that emit per-step partials on ring_walk_kernel,
+// 1 puts them on ring_walk64_kernel whenever the shapes allow (tests); unset, the chunk length decides
+static int walk64_partials_choice() {
   const char* e = std::getenv("RINGATTN_WIDE_PARTIALS");
-  return !(e && e[0] == '0');
+  return !e ? -1 : (e[0] == '0' ? 0 : 1);
 }
 
 struct ringattn_plan {
@@ -321,6 +323,10 @@ void push_segment(ringattn_plan* pl, TableSlice& slice, int q_start, int q_len,
   bool wide = true;
   for (size_t i = 0; i < items.size(); ++i) wide = wide && walk64_takes(pl->h_segitems[(size_t)sg.item_begin + i]);
   slice.wide = slice.seg_count == 0 ? wide : (slice.wide && wide);
+  for (size_t i = 0; i < items.size(); ++i) {
+    const int kv = pl->h_segitems[(size_t)sg.item_begin + i].kv_len;
+    slice.min_kv = (slice.seg_count == 0 && i == 0) ? kv : std::min(slice.min_kv, kv);
+  }
   ++slice.seg_count;
   slice.q_tiles_max = std::max(slice.q_tiles_max, q_tiles_of(q_len));
 }
@@ -448,8 +454,18 @@ int ensure_tables(ringattn_plan* pl) {
 
 // ring_walk64_kernel runs the launch of a slice when every KV range suits it and d = 128.  The launches that emit
 // partials go by the forward's ranges, so that the forward and the steps run one by one keep giving the same bits.
+// A chunk walked on its own costs ring_walk64_kernel a start and a drain of its pipeline, and its four waves move the
+// partials (stores, merge) more slowly than the eight of ring_walk_kernel.  It wins where its loop is well ahead --
+// causal forwards, whose masked tiles it skips wave by wave -- and the chunks are long; measured with per-step
+// partials, ring_walk64_kernel against ring_walk_kernel: cfg4 (causal, 4096 keys per chunk) 1130 against 1050
+// TFLOP/s, cfg5 (not causal, 8192) 1060 against 1145, cfg3 (not causal, 512) 590 against 700.
+constexpr int kWidePartialsMinKeys = 2048;
 bool slice_takes_walk64(const ringattn_plan* pl, const TableSlice& sl, int mode) {
-  if (mode != ringattn::kBlockCarryState && !(walk64_partials_enabled() && pl->fwd.wide)) return false;
+  if (mode != ringattn::kBlockCarryState) {
+    const int choice = walk64_partials_choice();
+    if (choice == 0 || !pl->fwd.wide) return false;
+    if (choice < 0 && !(pl->p.causal && pl->fwd.min_kv >= kWidePartialsMinKeys)) return false;
+  }
   return sl.wide && pl->p.dim == 128 && walk64_enabled();
 }
 

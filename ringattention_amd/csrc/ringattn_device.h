@@ -26,6 +26,12 @@ typedef short s16x8 __attribute__((ext_vector_type(8)));
 static __device__ __forceinline__ void load_lds_16(const void* base, int voff, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "m0");
 }
+// The same transfer for call sites whose base address may have just come out of a v_readfirstlane: a vector
+// instruction that wrote a scalar register must be five wait states ahead of the memory instruction that reads it,
+// and the compiler does not see into inline asm to provide them.
+static __device__ __forceinline__ void load_lds_16_settled(const void* base, int voff, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "m0");
+}
 static __device__ __forceinline__ unsigned lds_offset(const void* p) {
   return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
 }

@@ -26,6 +26,144 @@
 
 namespace ringattn {
 
+// Merge of the workgroup's 256 rows over the partials the workgroup has written (what merge_job_rows does for
+// ring_walk_kernel; the arithmetic and its order are merge_row's, so the bits are the merge kernel's).  With one wave
+// per SIMD nobody covers for a wave that waits for memory, so the partial rows are not fetched into registers a
+// batch at a time but streamed through LDS, which the rings have left free: every wave merges eight rows of each
+// group of 32 and keeps six blocks (eight rows of one part: 4 KB, 2 KB as fp16) in flight in a ring of its own,
+// with no barrier between the waves.  LDS: the partial LSEs [parts][256], the parts' first rows, the four rings.
+constexpr int kStagedMergeMaxParts = 24;  // LSEs of at most this many parts fit below the rings
+template <int DT, bool HP>
+static __device__ __forceinline__ void merge_rows_staged(const BlockArgs& a, const Segment& seg, int bh, int qt,
+                                                         unsigned char* smem, unsigned smem_base) {
+  constexpr int D = 128, BM = kWalkM;
+  constexpr int RB = HP ? D * 2 : D * 4;  // bytes per partial row
+  constexpr int SLOT = 8 * RB;            // a block: eight rows of one part
+  constexpr int LPB = SLOT / 1024;        // load instructions per block (1 KB per wave and instruction)
+  constexpr int NS = 6;                   // blocks in flight per wave
+  constexpr int PPR = RB / 16;            // 16-byte pieces per row
+  constexpr int NK = PPR / 8;             // pieces per lane and row
+  constexpr int CPP = HP ? 8 : 4;         // columns per piece
+  constexpr int kBaseAt = kStagedMergeMaxParts * BM * 4;  // behind the LSEs: the parts' first rows (int64 each)
+  constexpr int kRingAt = kBaseAt + 1024;  // (every 1 KB transfer stays inside a 1 KB block of LDS)
+  static_assert(kStagedMergeMaxParts * 8 <= 1024, "the parts' first rows fit");
+  static_assert(kRingAt + 4 * NS * SLOT <= 2 * 8 * 8192 + 8 * (kMaxParts + 4), "inside the kernel's LDS (rings and chunk list)");
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n_parts = seg.item_count;
+  const SegItem* its = a.items + seg.item_begin;
+  const int row0 = qt * BM;
+  const int rows_here = min(BM, seg.q_len - row0);
+  const int n_groups = (rows_here + 31) / 32;
+  float* lse_s = (float*)smem;
+  int64_t* base_s = (int64_t*)(smem + kBaseAt);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();  // the partial stores of all waves have completed and are visible to them; the LDS is idle
+  for (int i0 = 0; i0 < n_parts; i0 += 8) {  // thread tid: the LSEs of row tid
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (i0 + u < n_parts) {
+        const int64_t prow = its[i0 + u].part_base + (int64_t)bh * its[i0 + u].part_bh_stride + row0;
+        v[u] = tid < rows_here ? a.lse_part[prow + tid] : -INFINITY;
+        if (tid == 0) base_s[i0 + u] = prow;
+      }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (i0 + u < n_parts) lse_s[(i0 + u) * BM + tid] = v[u];
+  }
+  __syncthreads();
+
+  // block t = (group, part) in that order; this wave's rows of a group: 32 group + 8 wave + [0, 8)
+  const int total = n_groups * n_parts;
+  const unsigned ring = smem_base + kRingAt + wave * (NS * SLOT);
+  int ig = 0, ii = 0;  // group and part of the next block to issue
+  auto issue_block = [&](int slot) {
+    const int64_t prow = base_s[ii];
+    const uint64_t addr = (uint64_t)(uintptr_t)a.o_part + (uint64_t)prow * RB;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)addr), hi = __builtin_amdgcn_readfirstlane((unsigned)(addr >> 32));
+    const char* src = (const char*)(uintptr_t)(((uint64_t)hi << 32) | lo);  // row 0 of the job in part ii
+    const int r_first = 32 * ig + 8 * wave;
+#pragma unroll
+    for (int k = 0; k < LPB; ++k) {
+      const int pos = k * 64 + lane;  // 16-byte position within the block
+      const int r = pos / PPR, piece = (pos % PPR) ^ (8 * (r & 1));
+      const int rr = min(r_first + r, rows_here - 1);  // rows past the end of the segment: its last row again
+      load_lds_16_settled(src, rr * RB + piece * 16, ring + slot * SLOT + k * 1024);
+    }
+    if (++ii == n_parts) {
+      ii = 0;
+      ++ig;
+    }
+  };
+  for (int t = 0; t < NS && t < total; ++t) issue_block(t);
+
+  const int r8 = lane >> 3, c = lane & 7;
+  float mx = -INFINITY, wsum = 0.f, acc[NK * CPP];
+  int cg = 0, ci = 0;  // group and part of the block to consume
+  int slot = 0;
+  for (int t = 0; t < total; ++t) {
+    if (t + NS <= total) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 1) * LPB) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const int row = 32 * cg + 8 * wave + r8;  // within the job
+    f32x4 x[NK];
+    const unsigned char* blk = smem + kRingAt + wave * (NS * SLOT) + slot * SLOT + r8 * RB;
+#pragma unroll
+    for (int k = 0; k < NK; ++k) x[k] = *(const f32x4*)(blk + (((c + 8 * k) ^ (8 * (r8 & 1))) << 4));
+    if (ci == 0) {  // new rows: L = max over the parts first
+      mx = -INFINITY;
+      wsum = 0.f;
+#pragma unroll
+      for (int e = 0; e < NK * CPP; ++e) acc[e] = 0.f;
+      for (int i = 0; i < n_parts; ++i) mx = fmaxf(mx, lse_s[i * BM + row]);
+    }
+    const float L = lse_s[ci * BM + row];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the block is in registers: its slot takes the block NS further on
+    if (t + NS < total) issue_block(slot);
+    if (row < rows_here && L != -INFINITY) {  // (-inf: the identity element, its O may hold anything)
+      const float w = __expf(L - mx);
+      wsum += w;
+#pragma unroll
+      for (int k = 0; k < NK; ++k) {
+        if (HP) {
+          const f16x8 hv = __builtin_bit_cast(f16x8, x[k]);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[8 * k + e] = __builtin_fmaf(w, (float)hv[e], acc[8 * k + e]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[4 * k + e] = __builtin_fmaf(w, x[k][e], acc[4 * k + e]);
+        }
+      }
+    }
+    if (ci == n_parts - 1 && row < rows_here) {  // all parts in: normalise and store
+      if (mx != -INFINITY) {
+        const float inv = 1.f / wsum;
+#pragma unroll
+        for (int e = 0; e < NK * CPP; ++e) acc[e] *= inv;
+      }
+      const int64_t out_row = (int64_t)bh * a.S + seg.q_start + row0 + row;
+      typename Elem<DT>::type* orow = (typename Elem<DT>::type*)a.out + out_row * D;
+#pragma unroll
+      for (int k = 0; k < NK; ++k) {
+        if (HP) {
+          Store8<DT>::st(orow + (c + 8 * k) * 8, &acc[8 * k]);
+        } else {
+          typename Elem<DT>::vec4 o4;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o4[e] = (typename Elem<DT>::type)acc[4 * k + e];
+          *(typename Elem<DT>::vec4*)(orow + (c + 8 * k) * 4) = o4;
+        }
+      }
+      if (c == 0) a.lse[out_row] = (mx == -INFINITY) ? -INFINITY : mx + __logf(wsum);
+    }
+    if (++ci == n_parts) {
+      ci = 0;
+      ++cg;
+    }
+    slot = slot + 1 == NS ? 0 : slot + 1;
+  }
+}
+
 // KEEP: max / sum / acc-O run through all chunks of the q tile and the rows' result is written once (kBlockCarryState).
 // Otherwise the chunks are walked one by one, each as a sequence of its own -- prologue, loop, drain --, and each
 // ends in its normalised partial (O, LSE) (kBlockPartials, kBlockPartialsMerged; HP: partial O as fp16).
@@ -157,15 +295,15 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
   auto issue_k = [&](int slot) {
     const unsigned dst = __builtin_amdgcn_readfirstlane(smem_base + slot * TILE + 2 * wave * 1024);
     const char* p = k_head + __builtin_amdgcn_readfirstlane(kst.off);
-    load_lds_16(p, goff_k[0], dst);
-    load_lds_16(p, goff_k[1], dst + 1024);
+    load_lds_16_settled(p, goff_k[0], dst);
+    load_lds_16_settled(p, goff_k[1], dst + 1024);
     step(kst);
   };
   auto issue_v = [&](int slot) {
     const unsigned dst = __builtin_amdgcn_readfirstlane(smem_base + (NBUF + slot) * TILE + 2 * wave * 1024);
     const char* p = v_head + __builtin_amdgcn_readfirstlane(vst.off);
-    load_lds_16(p, goff_v[0], dst);
-    load_lds_16(p, goff_v[1], dst + 1024);
+    load_lds_16_settled(p, goff_v[0], dst);
+    load_lds_16_settled(p, goff_v[1], dst + 1024);
     step(vst);
   };
 
@@ -461,9 +599,13 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
     }
   }
   }  // passes
-  if (!KEEP && a.mode == kBlockPartialsMerged)  // this workgroup's rows over the partials it has just written
-    merge_job_rows<DT, D, HP, BM, 64 * WAVES>(a.o_part, a.lse_part, a.out, a.lse, a.items, seg, bh, qt, a.S,
-                                              (lds_float*)(__attribute__((address_space(3))) void*)smem);
+  if (!KEEP && a.mode == kBlockPartialsMerged) {  // this workgroup's rows over the partials it has just written
+    if (all_items <= kStagedMergeMaxParts)
+      merge_rows_staged<DT, HP>(a, seg, bh, qt, smem, smem_base);
+    else
+      merge_job_rows<DT, D, HP, BM, 64 * WAVES>(a.o_part, a.lse_part, a.out, a.lse, a.items, seg, bh, qt, a.S,
+                                                (lds_float*)(__attribute__((address_space(3))) void*)smem);
+  }
 }
 
 hipError_t launch_walk64(const BlockArgs& a, int dtype, hipStream_t stream) {

@@ -117,7 +117,8 @@ def test_chunk_by_chunk_walk_with_partials(oracle, w, half, monkeypatch):
     """The forward that keeps the ring steps apart (a partial (O, LSE) per chunk, merged at the end) on
     ring_walk64_kernel, which then walks every chunk as a sequence of its own: against the oracle, against the same
     forward on ring_walk_kernel (RINGATTN_WIDE_PARTIALS=0), and, bit for bit, against the steps launched one by one
-    with a separate merge."""
+    with a separate merge.  (RINGATTN_WIDE_PARTIALS=1: left to itself the library takes this kernel for per-step
+    partials only in causal forwards with at least 2048 keys per chunk.)"""
     q, k, v = rising_logits(w, 0.25) if w.name == "p_rise" else api.make_qkv_bits(w)
     qd, kd, vd = (api.bits_to_tensor(x, w.dtype) for x in (q, k, v))
 
@@ -139,7 +140,7 @@ def test_chunk_by_chunk_walk_with_partials(oracle, w, half, monkeypatch):
         return out, lse
 
     monkeypatch.delenv("RINGATTN_WIDE", raising=False)
-    monkeypatch.delenv("RINGATTN_WIDE_PARTIALS", raising=False)
+    monkeypatch.setenv("RINGATTN_WIDE_PARTIALS", "1")
     out_w, lse_w = run()
     check_rows(oracle, w, q, k, v, out_w, lse_w, np.arange(w.rows))
     monkeypatch.setenv("RINGATTN_WIDE_PARTIALS", "0")
@@ -150,3 +151,71 @@ def test_chunk_by_chunk_walk_with_partials(oracle, w, half, monkeypatch):
     ulp = 2.0 ** (np.floor(np.log2(np.maximum(big, 2.0 ** -14))) - mant)
     assert (np.abs(a - b) <= (3 if half else 2) * ulp).all()
     assert np.abs(lse_w.double().cpu().numpy() - lse_b.double().cpu().numpy()).max() <= 1e-4
+
+
+def test_first_launch_of_a_process_gives_the_bits_of_later_ones():
+    """A forward with per-step partials as the very first kernel of a fresh process (cold instruction cache and
+    address translation: the waves of a workgroup then drift apart as they never do later) against the same forward
+    repeated: bit for bit.  Four fresh processes."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import sys, torch\n"
+        "sys.path.insert(0, %r)\n"
+        "from ringattention_amd import api\n"
+        "from ringattention_amd.configs import Workload\n"
+        "w = Workload('first', 1, 3, 128, 4, 512, 'bf16', 71, False)\n"
+        "q, k, v = (api.bits_to_tensor(x, w.dtype) for x in api.make_qkv_bits(w))\n"
+        "plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, step_partials=True)\n"
+        "o1, l1 = plan.forward(q, k, v); torch.cuda.synchronize()\n"
+        "o2, l2 = plan.forward(q, k, v); torch.cuda.synchronize()\n"
+        "assert plan.forward_kernel() == 'ring_walk64_kernel'\n"
+        "assert torch.equal(o1.view(torch.int16), o2.view(torch.int16)) and torch.equal(l1, l2)\n" % root)
+    env = dict(os.environ, RINGATTN_WIDE_PARTIALS="1")
+    env.pop("RINGATTN_WIDE", None)
+    for _ in range(4):
+        r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+        assert r.returncode == 0, r.stderr[-2000:]
+
+
+def test_wide_partials_in_row_major_and_rank_local_buffers(monkeypatch):
+    """The chunk-by-chunk kernel writing caller-held partials: with a row's steps next to each other
+    (RINGATTN_FLAG_ROW_PARTIALS), and into one rank's buffers with heads no longer than a chunk of 256 rows (the load
+    streams then go round the head's first four tiles).  Bit for bit the forward that keeps its partials in the
+    workspace."""
+    monkeypatch.delenv("RINGATTN_WIDE", raising=False)
+    monkeypatch.setenv("RINGATTN_WIDE_PARTIALS", "1")
+    w = Workload("p_rows", 1, 2, 128, 4, 256, "bf16", 81, True)
+    q, k, v = (api.bits_to_tensor(x, w.dtype) for x in api.make_qkv_bits(w))
+    ref = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, step_partials=True)
+    out, lse = ref.forward(q, k, v)
+    assert ref.forward_kernel() == "ring_walk64_kernel"
+    ref.close()
+    plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, row_partials=True)
+    o_shape, l_shape = plan.parts_shapes()
+    o_parts = torch.zeros(o_shape, dtype=plan.part_dtype, device="cuda")
+    l_parts = torch.full(l_shape, float("-inf"), dtype=torch.float32, device="cuda")
+    for s in range(w.npes):
+        plan.block_forward(s, q, k, v, o_parts, l_parts)
+    out_r, lse_r = plan.merge_ring(o_parts, l_parts)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), out_r.view(torch.int16)) and torch.equal(lse, lse_r)
+    plan.close()
+    plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal)
+    c = w.chunk
+    for r in range(w.npes):
+        q_r = q[:, :, r * c:(r + 1) * c].contiguous()
+        o_shape, l_shape = plan.rank_parts_shapes(r)
+        o_parts = torch.zeros(o_shape, dtype=plan.part_dtype, device="cuda")
+        l_parts = torch.full(l_shape, float("-inf"), dtype=torch.float32, device="cuda")
+        for s in range(w.npes):
+            j = (r + s) % w.npes
+            plan.rank_step_forward(r, s, q_r, k[:, :, j * c:(j + 1) * c].contiguous(), v[:, :, j * c:(j + 1) * c].contiguous(),
+                                   o_parts[s], l_parts[s])
+        o_r, l_r = plan.rank_merge(r, o_parts, l_parts)
+        torch.cuda.synchronize()
+        assert torch.equal(o_r.view(torch.int16), out[:, :, r * c:(r + 1) * c].view(torch.int16)), f"rank {r}"
+        assert torch.equal(l_r, lse[:, :, r * c:(r + 1) * c]), f"rank {r}"
+    plan.close()
