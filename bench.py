@@ -34,10 +34,10 @@ PEAK_HBM_GBS = 8000.0
 # (bytes, summary under profiles/, kernel, kernel_source_id(kernel) when it was measured).  The figure is only printed
 # while the forward still runs that kernel and its source is still the one that was profiled.
 MEASURED_TRAFFIC = {
-    "cfg4": (2260e6, "profiles/ring_walk64_kernel_cfg4.md", "ring_walk64_kernel", "@W64@"),
-    "cfg3": (2354e6, "profiles/ring_walk64_kernel_other_workloads.md", "ring_walk64_kernel", "@W64@"),
-    "cfg5": (43590e6, "profiles/ring_walk64_kernel_other_workloads.md", "ring_walk64_kernel", "@W64@"),
-    "cfg2": (34.3e6, "profiles/ring_walk_kernel_other_workloads.md", "ring_walk_kernel", "494a183db25c449b"),
+    "cfg4": (2243e6, "profiles/ring_walk64_kernel_cfg4.md", "ring_walk64_kernel", "da96d76e590da0fa"),
+    "cfg3": (2322e6, "profiles/ring_walk64_kernel_other_workloads.md", "ring_walk64_kernel", "da96d76e590da0fa"),
+    "cfg5": (40750e6, "profiles/ring_walk64_kernel_other_workloads.md", "ring_walk64_kernel", "da96d76e590da0fa"),
+    "cfg2": (34.3e6, "profiles/ring_walk_kernel_other_workloads.md", "ring_walk_kernel", "88c93081e9f9f570"),
 }
 KERNEL_SOURCES = {
     "ring_walk64_kernel": ("ringattn_walk64.hip", "ringattn_walk64_loop.inc", "ringattn_device.h"),

@@ -1,8 +1,9 @@
 // gfx950 (CDNA4) kernel: block attention over the ring steps of 256 query rows, 64 rows per wave.
 //
-//   ring_walk64_kernel : the carried-state forward of ring_walk_kernel (ringattn_walk.hip; the
-//       reference's CTA that walks its ring steps with max / sum / acc-O in registers,
-//       csrc/ring_attention.cu:439-443,456-620, epilogue :621-664) for d = 128, laid out for ONE wave
+//   ring_walk64_kernel : the forward of ring_walk_kernel (ringattn_walk.hip; the reference's CTA
+//       that walks its ring steps with max / sum / acc-O in registers,
+//       csrc/ring_attention.cu:439-443,456-620, epilogue :621-664; or, chunk by chunk, with a partial
+//       (O, LSE) per ring step and their merge at the end) for d = 128, laid out for ONE wave
 //       per SIMD: a workgroup of FOUR waves owns the same 256 query rows, each wave two 32-query
 //       blocks.  Every K fragment and every V^T fragment read from LDS then feeds two MFMAs (one per
 //       block) instead of one: half the LDS fragment traffic per MFMA.  With 512 registers per wave
