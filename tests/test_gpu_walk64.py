@@ -154,9 +154,9 @@ def test_chunk_by_chunk_walk_with_partials(oracle, w, half, monkeypatch):
 
 
 def test_first_launch_of_a_process_gives_the_bits_of_later_ones():
-    """A forward with per-step partials as the very first kernel of a fresh process (cold instruction cache and
-    address translation: the waves of a workgroup then drift apart as they never do later) against the same forward
-    repeated: bit for bit.  Four fresh processes."""
+    """A forward as the very first kernel of a fresh process (cold instruction cache and address translation: the waves
+    of a workgroup then drift apart as they never do later) against the same forward repeated: bit for bit.  Four fresh
+    processes, two with per-step partials and two with the state carried."""
     import os
     import subprocess
     import sys
@@ -166,17 +166,18 @@ def test_first_launch_of_a_process_gives_the_bits_of_later_ones():
         "sys.path.insert(0, %r)\n"
         "from ringattention_amd import api\n"
         "from ringattention_amd.configs import Workload\n"
-        "w = Workload('first', 1, 3, 128, 4, 512, 'bf16', 71, False)\n"
+        "partials = sys.argv[1] == '1'\n"
+        "w = Workload('first', 1, 3, 128, 4, 512, 'bf16', 71, not partials)\n"
         "q, k, v = (api.bits_to_tensor(x, w.dtype) for x in api.make_qkv_bits(w))\n"
-        "plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, step_partials=True)\n"
+        "plan = api.RingAttention(w.npes, w.chunk, w.dim, w.batch, w.heads, w.dtype, w.causal, step_partials=partials)\n"
         "o1, l1 = plan.forward(q, k, v); torch.cuda.synchronize()\n"
         "o2, l2 = plan.forward(q, k, v); torch.cuda.synchronize()\n"
         "assert plan.forward_kernel() == 'ring_walk64_kernel'\n"
         "assert torch.equal(o1.view(torch.int16), o2.view(torch.int16)) and torch.equal(l1, l2)\n" % root)
     env = dict(os.environ, RINGATTN_WIDE_PARTIALS="1")
     env.pop("RINGATTN_WIDE", None)
-    for _ in range(4):
-        r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    for partials in ("1", "0", "1", "0"):
+        r = subprocess.run([sys.executable, "-c", code, partials], env=env, capture_output=True, text=True, timeout=110)
         assert r.returncode == 0, r.stderr[-2000:]
 
 
