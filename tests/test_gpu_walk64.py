@@ -220,3 +220,58 @@ def test_wide_partials_in_row_major_and_rank_local_buffers(monkeypatch):
         assert torch.equal(o_r.view(torch.int16), out[:, :, r * c:(r + 1) * c].view(torch.int16)), f"rank {r}"
         assert torch.equal(l_r, lse[:, :, r * c:(r + 1) * c]), f"rank {r}"
     plan.close()
+
+
+def test_random_wide_plans_against_oracle(oracle, monkeypatch):
+    """A seeded sweep over the shapes ring_walk64_kernel takes: 1 to 8 ranks of 128 to 1024 tokens each (multiples of
+    32, unequal), batch, grouped heads, both types, the causal mask in both layouts, an explicit scale, graph replay, the
+    state carried or per-step partials (on this kernel: RINGATTN_WIDE_PARTIALS=1).  Every plan must report this kernel;
+    up to 3000 rows of each (the first and the last q tile of a head, chunk edges, random ones) against the oracle."""
+    monkeypatch.delenv("RINGATTN_WIDE", raising=False)
+    monkeypatch.setenv("RINGATTN_WIDE_PARTIALS", "1")
+    rng = np.random.default_rng(4242)
+    for case in range(60):
+        P = int(rng.integers(1, 9))
+        causal = bool(rng.integers(0, 2))
+        zigzag = causal and bool(rng.integers(0, 2))
+        lens = [32 * int(rng.integers(4, 33)) for _ in range(P)]
+        if zigzag:
+            lens = [64 * max(4, c // 64) for c in lens]      # both halves of a rank: multiples of 32, at least 128
+        dtype = str(rng.choice(["fp16", "bf16"]))
+        B, hkv, group = int(rng.integers(1, 3)), int(rng.integers(1, 3)), int(rng.integers(1, 3))
+        H, S = hkv * group, sum(lens)
+        scale = float(rng.choice([0.0, 0.0, 0.05]))
+        graph = bool(rng.integers(0, 2))
+        steps_apart = case % 3 == 2
+        tag = (f"case {case}: P={P} lens={lens} B={B} H={H} hkv={hkv} {dtype} causal={causal} zigzag={zigzag} "
+               f"scale={scale} graph={graph} step_partials={steps_apart}")
+        print(tag, flush=True)
+        w = Workload("wide_rand", B, H, 128, 1, S, dtype, 3000 + case, causal)
+        q, _, _ = api.make_qkv_bits(w)
+        _, k, v = api.make_qkv_bits(Workload("wide_rand_kv", B, hkv, 128, 1, S, dtype, 4000 + case, causal))
+        order = api.zigzag_order(lens) if zigzag else np.arange(S)
+        inv = torch.from_numpy(np.argsort(order)).cuda()
+        qd, kd, vd = (api.bits_to_tensor(np.ascontiguousarray(x[:, :, order]), dtype) for x in (q, k, v))
+        plan = api.RingAttention(P, lens, 128, B, H, dtype, causal, softmax_scale=scale, graph=graph,
+                                 kv_heads=hkv if group > 1 else 0, layout="zigzag" if zigzag else "contiguous",
+                                 step_partials=steps_apart)
+        try:
+            assert plan.forward_kernel() == "ring_walk64_kernel", tag
+            out, lse = plan.forward(qd, kd, vd)
+            if graph:
+                out2, lse2 = plan.forward(qd, kd, vd, torch.empty_like(out), torch.empty_like(lse))
+                torch.cuda.synchronize()
+                assert torch.equal(out, out2) and torch.equal(lse, lse2), tag
+            torch.cuda.synchronize()
+        finally:
+            plan.close()
+        rows = np.arange(w.rows)
+        if len(rows) > 3000:
+            head = rows[:S]
+            edges = np.concatenate([np.cumsum(lens)[:-1] + o for o in (-1, 0, 1)]) if P > 1 else np.zeros(0, int)
+            pick = np.concatenate([head[:256], head[-256:], edges, (B * H - 1) * S + head[-256:],
+                                   rng.choice(rows, 2000, replace=False)])
+            rows = np.unique(pick.astype(np.int64))
+        k_full, v_full = (np.repeat(x, group, axis=1) for x in (k, v))
+        check_rows(oracle, w, q, k_full, v_full, out[:, :, inv].contiguous(), lse[:, :, inv].contiguous(), rows,
+                   scale=scale if scale > 0 else None)
