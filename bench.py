@@ -40,7 +40,7 @@ MEASURED_TRAFFIC = {
     "cfg2": (34.3e6, "profiles/ring_walk_kernel_other_workloads.md", "ring_walk_kernel", "88c93081e9f9f570"),
 }
 KERNEL_SOURCES = {
-    "ring_walk64_kernel": ("ringattn_walk64.hip", "ringattn_walk64_loop.inc", "ringattn_device.h"),
+    "ring_walk64_kernel": ("ringattn_walk64.hip", "ringattn_walk64_loop.inc", "ringattn_walk64_loop_d64.inc", "ringattn_device.h"),
     "ring_walk_kernel": ("ringattn_walk.hip", "ringattn_device.h"),
 }
 BASELINE_METRIC = "ring-attn fwd TFLOP/s + % bf16 MFMA peak, S=32K d=128 8-step ring, 1 GPU"

@@ -56,6 +56,7 @@ def source_id(paths):
 def library_sources():
     return [os.path.join(CSRC, s) for s in SOURCES] + [os.path.join(CSRC, "ringattn_kernels.h"), os.path.join(CSRC, "ringattn_device.h"),
                                                        os.path.join(CSRC, "ringattn_walk64_loop.inc"),
+                                                       os.path.join(CSRC, "ringattn_walk64_loop_d64.inc"),
                                                        os.path.join(REPO_DIR, "include", "ringattn.h")]
 
 

@@ -2,8 +2,8 @@
 """Generates ringattn_walk64_loop.inc: the steady loop of ring_walk64_kernel (ringattn_walk64.hip) as ONE
 inline-assembly statement with hand-allocated registers and a hand-made instruction order.
 
-    python3 gen_walk64_loop.py            # rewrites ringattn_walk64_loop.inc next to this file
-    python3 gen_walk64_loop.py --check    # exit status 1 if the committed file differs
+    python3 gen_walk64_loop.py            # rewrites ringattn_walk64_loop.inc (d = 128) and ringattn_walk64_loop_d64.inc next to this file
+    python3 gen_walk64_loop.py --check    # exit status 1 if a committed file differs
 
 Why by hand: one wave per SIMD has nobody to hide behind.  Within an iteration the matrix work (S(u+1) = K(u+1) Q^T
 and O += P(u-1) V(u-1) for both 32-query blocks of the wave: 32 MFMAs) and the vector work (P(u) = exp2(S(u) k2 - m k2),
@@ -12,7 +12,10 @@ issued evenly interleaved (one MFMA, then four or five vector instructions) with
 MFMAs ahead of its use.  The compiler, given the same loop as C++, keeps Q in AccVGPRs and copies it back for every
 MFMA, serialises the fragment reads behind waits and puts the exponentials after the MFMAs.
 
-Register map (fixed; the C++ side hands its values over in exactly these registers):
+At d = 64 a tile has half the MFMAs (16) for the same vector work, seven to eight vector instructions go behind each, a
+K or V tile is 4 KB (one 1 KB piece per wave), acc-O takes a[0:63] and Q a[64:95]; everything else is the same text.
+
+Register map (d = 128; fixed; the C++ side hands its values over in exactly these registers):
     a[0:127]    acc-O: block b, head-dim block db at a[64 b + 16 db .. +15]
     a[128:191]  Q (B operands): block b, slice ks at a[128 + 32 b + 4 ks .. +3]
     v[0:63]     scores, two buffers of 2 x 16: buffer f, block b at v[32 f + 16 b .. +15]; exponentials are taken in place
@@ -34,21 +37,37 @@ def _knob(name, default):
     return int(os.environ.get("W64_" + name, default))
 
 
-TILE = 8192
 NBUF = 8
-ROWB = 256
 UNROLL = 8      # iterations per trip: ring slots are immediates
 LEAD = _knob('LEAD', 3)        # a fragment read is issued this many MFMAs ahead of the MFMA that needs it
 HEAD_VALU = _knob('HEAD', 4)   # vector instructions in front of the first MFMA of an iteration
 PREREAD = _knob('PREREAD', 4)     # K fragments of the next iteration read at the end of this one
 
 
+def configure(d):
+    """The head dimension the text is generated for."""
+    global D, KS, DB, ROWB, TILE, PIECES, LOADS_IN_FLIGHT, SHARE, MASK_AT
+    D = d
+    KS, DB = d // 16, d // 32          # contraction slices of QK^T, 32-wide blocks of the head dim in PV
+    ROWB = 2 * d                       # bytes per row
+    TILE = 32 * ROWB                   # bytes per tile
+    PIECES = TILE // 4096              # 1 KB pieces of a tile per wave
+    LOADS_IN_FLIGHT = 3 * 2 * PIECES   # at the barrier: the loads of the last three iterations (two tiles each)
+    # vector instructions behind an even / odd MFMA
+    SHARE = (_knob('SHARE_A', 3), _knob('SHARE_B', 4)) if d == 128 else (_knob('SHARE_A', 7), _knob('SHARE_B', 8))
+    MASK_AT = 2 * KS + 3    # the mask of tile u+1 is applied (if at all) behind this MFMA: the last QK MFMA is index 2 KS - 1
+
+
+configure(128)
+
+
 def O(b, db):
-    return "a[%d:%d]" % (64 * b + 16 * db, 64 * b + 16 * db + 15)
+    return "a[%d:%d]" % (16 * (DB * b + db), 16 * (DB * b + db) + 15)
 
 
 def Q(b, ks):
-    return "a[%d:%d]" % (128 + 32 * b + 4 * ks, 128 + 32 * b + 4 * ks + 3)
+    base = 32 * DB + 4 * (KS * b + ks)
+    return "a[%d:%d]" % (base, base + 3)
 
 
 def Sreg(f, b, e):
@@ -103,7 +122,6 @@ S_KHEAD, S_VHEAD = (44, 45), (46, 47)
 S_K2, S_LDSK, S_LDSV = "s48", "s49", "s50"
 S_C, S_STOP, S_FAR, S_MW1, S_N = "s51", "s52", "s53", "s54", "s55"
 S_T = lambda i: "s%d" % (56 + i)
-MASK_AT = 19    # the mask of tile u+1 is applied (if at all) behind this MFMA: the last QK MFMA is index 15
 VLIM = lambda b: "v%d" % (190 + b)
 
 
@@ -128,23 +146,30 @@ _redo = []    # (label number, score buffer) of every place the speculative expo
 
 
 def tile_load(st, slot, goff):
-    """Both pieces of one tile, then the step of the stream to the next tile (the change of chunk is out of line)."""
+    """The pieces of one tile this wave loads, then the step of the stream to the next tile (the change of chunk is out
+    of line)."""
     site = len(_sites)
     _sites.append((site, st))
     ld = "s_nop 0 ;" if _knob('NOLOADS', 0) else ""   # timing only
-    return [
+    out = [
         "s_add_u32 m0, %s, %d" % (st.lds, slot * TILE),
         "s_sub_u32 %s, %s, 1" % (st.left, st.left),
         ld + "global_load_lds_dwordx4 %s, %s" % (goff(0), st.ptr),
-        "s_add_u32 m0, %s, %d" % (st.lds, slot * TILE + 1024),
-        "s_nop 0",
-        ld + "global_load_lds_dwordx4 %s, %s" % (goff(1), st.ptr),
+    ]
+    if PIECES == 2:
+        out += [
+            "s_add_u32 m0, %s, %d" % (st.lds, slot * TILE + 1024),
+            "s_nop 0",
+            ld + "global_load_lds_dwordx4 %s, %s" % (goff(1), st.ptr),
+        ]
+    out += [
         "s_add_u32 %s, %s, %d" % (st.lo, st.lo, TILE),
         "s_addc_u32 %s, %s, 0" % (st.hi, st.hi),
         "s_cmp_eq_u32 %s, 0" % st.left,
         "s_cbranch_scc1 3%02df" % site,
         "4%02d:" % site,
     ]
+    return out
 
 
 def chunk_changes():
@@ -169,7 +194,7 @@ def chunk_changes():
 def k_prereads(i_next):
     """The first K fragments of iteration i_next (tile u+1 of that iteration)."""
     slot = (i_next + 1) % NBUF
-    return ["ds_read_b128 %s, %s offset:%d" % (KF(ks), KOFF(ks), slot * TILE) for ks in range(PREREAD)]
+    return ["ds_read_b128 %s, %s offset:%d" % (KF(ks), KOFF(ks), slot * TILE) for ks in range(min(PREREAD, KS))]
 
 
 def exp_stream(cur, cvt):
@@ -236,14 +261,15 @@ def redo_routine(cur, cvt):
         for q in range(4):
             out.append("v_mul_f32 %s, %s, %s" % (LS(b, q), LS(b, q), TMP(6 + b)))
     # acc-O, eight registers at a time through the (dead) exponential buffer
+    per_block = 16 * DB
     for b in range(2):
-        for r0 in range(0, 64, 8):
+        for r0 in range(0, per_block, 8):
             for r in range(8):
-                out.append("v_accvgpr_read_b32 %s, a%d" % (PX(0, r), 64 * b + r0 + r))
+                out.append("v_accvgpr_read_b32 %s, a%d" % (PX(0, r), per_block * b + r0 + r))
             for r in range(8):
                 out.append("v_mul_f32 %s, %s, %s" % (PX(0, r), PX(0, r), TMP(6 + b)))
             for r in range(8):
-                out.append("v_accvgpr_write_b32 a%d, %s" % (64 * b + r0 + r, PX(0, r)))
+                out.append("v_accvgpr_write_b32 a%d, %s" % (per_block * b + r0 + r, PX(0, r)))
     out += exp_stream(cur, cvt)
     for site, c in _redo:
         if c == cur:
@@ -263,7 +289,7 @@ def iteration(i, mfma, cvt, do_qk=True, do_sm=True, do_pv=True):
     # barrier ago; the V fragments of this iteration are only read behind this barrier.
     misc = []
     if i % 2 == 0:
-        misc += ["s_waitcnt vmcnt(12)"] + ([] if _knob('NOBARRIER', 0) else ["s_barrier"])
+        misc += ["s_waitcnt vmcnt(%d)" % LOADS_IN_FLIGHT] + ([] if _knob('NOBARRIER', 0) else ["s_barrier"])
         misc += tile_load(KST, (i + 7) % NBUF, GOFFK)
         misc += tile_load(KST, i % NBUF, GOFFK)
     else:
@@ -277,15 +303,15 @@ def iteration(i, mfma, cvt, do_qk=True, do_sm=True, do_pv=True):
     mf = []   # (text, index of the last fragment read it needs)
     reads = []  # fragment reads in the order they are issued
     if do_qk:
-        for ks in range(8):
+        for ks in range(KS):
             reads.append("ds_read_b128 %s, %s offset:%d" % (KF(ks), KOFF(ks), kslot * TILE))
             for b in range(2):
                 src_c = "0" if ks == 0 else Svec(nxt, b)
                 mf.append(("%s %s, %s, %s, %s" % (mfma, Svec(nxt, b), KF(ks), Q(b, ks), src_c), len(reads) - 1))
     n_qk = len(mf)
     for t2 in (range(2) if do_pv else ()):
-        for db in range(4):
-            idx = 4 * t2 + db
+        for db in range(DB):
+            idx = DB * t2 + db
             off = vslot * TILE + 16 * t2 * ROWB
             reads.append("ds_read_b64_tr_b16 %s, %s offset:%d" % (VFlo(idx), VOFF(db), off))
             reads.append("ds_read_b64_tr_b16 %s, %s offset:%d" % (VFhi(idx), VOFF(db), off + 8 * ROWB))
@@ -313,7 +339,7 @@ def iteration(i, mfma, cvt, do_qk=True, do_sm=True, do_pv=True):
             valu.append("v_subrev_u32_e32 %s, 32, %s" % (VLIM(b), VLIM(b)))
 
     # ---- interleave
-    issued = PREREAD if do_qk else 0   # the first K fragments are on their way (read at the end of the previous iteration)
+    issued = min(PREREAD, KS) if do_qk else 0   # the first K fragments are on their way (read at the end of the previous iteration)
     if not do_qk:
         out.append("s_waitcnt lgkmcnt(0)")   # K fragments read ahead for a product that does not take place
 
@@ -350,7 +376,7 @@ def iteration(i, mfma, cvt, do_qk=True, do_sm=True, do_pv=True):
             out += ["s_cmp_ge_i32 %s, %s" % (S_C, S_MW1), "s_cbranch_scc1 5%d0f" % i, "6%d0:" % i]
             masked = True
             spent += 8
-        share = _knob('SHARE_A', 3) if j % 2 == 0 else _knob('SHARE_B', 4)
+        share = SHARE[j % 2]
         n_here = 0
         if MISC_AT and j + 1 >= MISC_AT:
             take = _knob('MISC_N', 3)
@@ -444,7 +470,7 @@ def loop_text(mfma, cvt):
 def operands():
     outs, ins = [], []
     for b in range(2):
-        for db in range(4):
+        for db in range(DB):
             outs.append('"+{%s}"(oacc[%d][%d])' % (O(b, db), b, db))
     for b in range(2):
         outs.append('"+{%s}"(sacc[%d])' % (Svec(0, b), b))
@@ -465,15 +491,15 @@ def operands():
     for b in range(2):
         outs.append('"+{%s}"(vlim[%d])' % (VLIM(b), b))
     for b in range(2):
-        for ks in range(8):
+        for ks in range(KS):
             ins.append('"{%s}"(qf[%d][%d])' % (Q(b, ks), b, ks))
-    for ks in range(8):
+    for ks in range(KS):
         ins.append('"{%s}"(koff_a[%d])' % (KOFF(ks), ks))
-    for db in range(4):
+    for db in range(DB):
         ins.append('"{%s}"(voff_a[%d])' % (VOFF(db), db))
-    for j in range(2):
+    for j in range(PIECES):
         ins.append('"{%s}"(goff_k[%d])' % (GOFFK(j), j))
-    for j in range(2):
+    for j in range(PIECES):
         ins.append('"{%s}"(goff_v[%d])' % (GOFFV(j), j))
     ins += ['"{%s}"(kh_lo)' % KST.head[0], '"{%s}"(kh_hi)' % KST.head[1], '"{%s}"(vh_lo)' % VST.head[0], '"{%s}"(vh_hi)' % VST.head[1],
             '"{%s}"(k2_bits)' % S_K2, '"{%s}"(lds_dst_k)' % S_LDSK, '"{%s}"(lds_dst_v)' % S_LDSV,
@@ -483,7 +509,8 @@ def operands():
     return outs, ins, clob
 
 
-def render():
+def render(d=128):
+    configure(d)
     res = ["// Generated by gen_walk64_loop.py -- do not edit.  The steady loop of ring_walk64_kernel: see the generator for the",
            "// register map and the instruction order.  Expects the kernel's variables by name.", ""]
     for dt, (mfma, cvt) in enumerate((("v_mfma_f32_32x32x16_f16", "v_cvt_pk_f16_f32"),
@@ -500,12 +527,21 @@ def render():
     return "\n".join(res) + "\n"
 
 
+FILES = {128: "ringattn_walk64_loop.inc", 64: "ringattn_walk64_loop_d64.inc"}
+
 if __name__ == "__main__":
-    path = os.environ.get("W64_OUT") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "ringattn_walk64_loop.inc")
-    text = render()
-    if "--check" in sys.argv:
-        with open(path) as f:
-            sys.exit(0 if f.read() == text else 1)
-    with open(path, "w") as f:
-        f.write(text)
-    print("wrote", path, len(text.split("\n")), "lines")
+    here = os.environ.get("W64_OUT_DIR") or os.path.dirname(os.path.abspath(__file__))
+    status = 0
+    for d, name in FILES.items():
+        path = os.path.join(here, name)
+        if d == 128 and os.environ.get("W64_OUT"):
+            path = os.environ["W64_OUT"]
+        text = render(d)
+        if "--check" in sys.argv:
+            with open(path) as f:
+                status |= 0 if f.read() == text else 1
+            continue
+        with open(path, "w") as f:
+            f.write(text)
+        print("wrote", path, len(text.split("\n")), "lines")
+    sys.exit(status)

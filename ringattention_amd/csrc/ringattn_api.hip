@@ -220,6 +220,11 @@ static bool walk64_enabled() {
 }
 // RINGATTN_WIDE_PARTIALS in the environment: 0 keeps the launches that emit per-step partials on ring_walk_kernel,
 // 1 puts them on ring_walk64_kernel whenever the shapes allow (tests); unset, the chunk length decides
+// RINGATTN_WIDE_D64=0 keeps the d = 64 forwards (state carried) on ring_walk_kernel
+static bool walk64_d64_enabled() {
+  const char* e = std::getenv("RINGATTN_WIDE_D64");
+  return !(e && e[0] == '0');
+}
 static int walk64_partials_choice() {
   const char* e = std::getenv("RINGATTN_WIDE_PARTIALS");
   return !e ? -1 : (e[0] == '0' ? 0 : 1);
@@ -461,12 +466,14 @@ int ensure_tables(ringattn_plan* pl) {
 // TFLOP/s, cfg5 (not causal, 8192) 1060 against 1145, cfg3 (not causal, 512) 590 against 700.
 constexpr int kWidePartialsMinKeys = 2048;
 bool slice_takes_walk64(const ringattn_plan* pl, const TableSlice& sl, int mode) {
+  if (!sl.wide || !walk64_enabled()) return false;
   if (mode != ringattn::kBlockCarryState) {
     const int choice = walk64_partials_choice();
-    if (choice == 0 || !pl->fwd.wide) return false;
+    if (pl->p.dim != 128 || choice == 0 || !pl->fwd.wide) return false;
     if (choice < 0 && !(pl->p.causal && pl->fwd.min_kv >= kWidePartialsMinKeys)) return false;
+    return true;
   }
-  return sl.wide && pl->p.dim == 128 && walk64_enabled();
+  return pl->p.dim == 128 || (pl->p.dim == 64 && walk64_d64_enabled());
 }
 
 // A block launch over a slice of the tables.
@@ -477,7 +484,7 @@ int launch_slice(const ringattn_plan* pl, const TableSlice& sl, ringattn::BlockA
   a.n_segs = sl.seg_count;
   a.q_tiles_max = sl.q_tiles_max;
   if (slice_takes_walk64(pl, sl, a.mode))
-    RA_HIP(ringattn::launch_walk64(a, pl->p.dtype, stream));
+    RA_HIP(ringattn::launch_walk64(a, pl->p.dtype, pl->p.dim, stream));
   else
     RA_HIP(ringattn::launch_walk(a, pl->p.dtype, pl->p.dim, stream));
   return RINGATTN_OK;
@@ -611,9 +618,9 @@ int run_rank_call(const RankCall& rc, void* scratch, const void* q, const void* 
   a.q_tiles_max = q_tiles_of(c);
   a.bh_stride = (int64_t)c * dim;  // q and out hold this rank's rows only; k and v the whole sequence
   a.S = c;
-  bool wide = dim == 128 && walk64_enabled();
+  bool wide = (dim == 128 || (dim == 64 && walk64_d64_enabled())) && walk64_enabled();
   for (int i = 0; i < n_parts; ++i) wide = wide && walk64_takes(rc.pack.items[i]);
-  if (wide) RA_HIP(ringattn::launch_walk64(a, rc.p.dtype, stream));
+  if (wide) RA_HIP(ringattn::launch_walk64(a, rc.p.dtype, dim, stream));
   else RA_HIP(ringattn::launch_walk(a, rc.p.dtype, dim, stream));
   return RINGATTN_OK;
 }

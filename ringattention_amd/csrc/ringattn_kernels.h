@@ -123,7 +123,7 @@ struct TablePack {
 hipError_t launch_walk(const BlockArgs& a, int dtype, int dim, hipStream_t stream);  // ring_walk_kernel, any BlockMode
 // ring_walk64_kernel: the carried-state forward at d = 128 with 64 query rows per wave; only for tables that
 // walk64_takes() accepts
-hipError_t launch_walk64(const BlockArgs& a, int dtype, hipStream_t stream);
+hipError_t launch_walk64(const BlockArgs& a, int dtype, int dim, hipStream_t stream);
 hipError_t launch_merge(const MergeArgs& a, int dtype, int dim, hipStream_t stream);
 // writes pack.seg to *seg_dst and pack.items[0..n) to item_dst
 hipError_t launch_write_table(const TablePack& pack, int n, Segment* seg_dst, SegItem* item_dst, hipStream_t stream);

@@ -168,10 +168,12 @@ static __device__ __forceinline__ void merge_rows_staged(const BlockArgs& a, con
 // KEEP: max / sum / acc-O run through all chunks of the q tile and the rows' result is written once (kBlockCarryState).
 // Otherwise the chunks are walked one by one, each as a sequence of its own -- prologue, loop, drain --, and each
 // ends in its normalised partial (O, LSE) (kBlockPartials, kBlockPartialsMerged; HP: partial O as fp16).
-template <int DT, bool KEEP, bool HP>
+// D = 64 (state carried only): half the MFMAs per tile for the same vector work, 4 KB tiles (one 1 KB piece per wave),
+// 64 KB of rings.
+template <int DT, int D, bool KEEP, bool HP>
 __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) {
   using E = Elem<DT>;
-  constexpr int D = 128;
+  static_assert(D == 128 || (D == 64 && KEEP && !HP), "d = 64 is built with the state carried only");
   constexpr int WAVES = 4;
   constexpr int BM = kWalkM;       // query rows per workgroup: 4 waves x 64
   constexpr int BN = 32;           // keys per tile
@@ -179,6 +181,7 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
   constexpr int CPR = D / 8;       // 16-byte chunks per row
   constexpr int ROWB = D * 2;      // bytes per row
   constexpr int TILE = BN * ROWB;  // bytes per tile
+  constexpr int PIECES = TILE / 4096;  // 1 KB pieces of a tile per wave
   constexpr int KS = D / 16;       // contraction slices of QK^T
   constexpr int DB = D / 32;       // 32-wide blocks of the head dim in PV
   constexpr float kLazyLog2 = 8.f;
@@ -218,11 +221,11 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qf[b][ks] = *(const s16x8*)(qrow + ks * 32);
   }
-  // the two 1 KB pieces of a tile this wave loads (pieces 2 wave and 2 wave + 1 of eight)
-  int goff_k[2], goff_v[2];
+  // the 1 KB pieces of a tile this wave loads (d = 128: pieces 2 wave and 2 wave + 1 of eight; d = 64: piece wave of four)
+  int goff_k[PIECES], goff_v[PIECES];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int pk = (2 * wave + j) * 64 + lane;
+  for (int j = 0; j < PIECES; ++j) {
+    const int pk = (PIECES * wave + j) * 64 + lane;
     goff_k[j] = (pk / CPR) * ROWB + (((pk % CPR) ^ k_swizzle<D>(pk / CPR)) << 4);
     goff_v[j] = (pk / CPR) * ROWB + (((pk % CPR) ^ v_swizzle<D>(pk / CPR)) << 4);
   }
@@ -294,17 +297,17 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
   chunk_of(0, kst.off, kst.left);
   chunk_of(0, vst.off, vst.left);
   auto issue_k = [&](int slot) {
-    const unsigned dst = __builtin_amdgcn_readfirstlane(smem_base + slot * TILE + 2 * wave * 1024);
+    const unsigned dst = __builtin_amdgcn_readfirstlane(smem_base + slot * TILE + PIECES * wave * 1024);
     const char* p = k_head + __builtin_amdgcn_readfirstlane(kst.off);
-    load_lds_16_settled(p, goff_k[0], dst);
-    load_lds_16_settled(p, goff_k[1], dst + 1024);
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) load_lds_16_settled(p, goff_k[j], dst + 1024 * j);
     step(kst);
   };
   auto issue_v = [&](int slot) {
-    const unsigned dst = __builtin_amdgcn_readfirstlane(smem_base + (NBUF + slot) * TILE + 2 * wave * 1024);
+    const unsigned dst = __builtin_amdgcn_readfirstlane(smem_base + (NBUF + slot) * TILE + PIECES * wave * 1024);
     const char* p = v_head + __builtin_amdgcn_readfirstlane(vst.off);
-    load_lds_16_settled(p, goff_v[0], dst);
-    load_lds_16_settled(p, goff_v[1], dst + 1024);
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) load_lds_16_settled(p, goff_v[j], dst + 1024 * j);
     step(vst);
   };
 
@@ -434,9 +437,10 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
     return __builtin_amdgcn_ballot_w64(far) != 0;
   };
   // the barrier of a pair of iterations: every wave's loads of four and more iterations ago have landed (each
-  // iteration issues four); the loads of the last three stay in flight
+  // iteration issues two tiles: 2 PIECES loads); the loads of the last three stay in flight
   auto ring_barrier = [&]() {
-    asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    if (PIECES == 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
     __syncthreads();
   };
 
@@ -491,8 +495,8 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
   }
   {
     f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-    *(f32x4*)(smem + (NBUF + 7) * TILE + tid * 32) = zero;
-    *(f32x4*)(smem + (NBUF + 7) * TILE + tid * 32 + 16) = zero;
+#pragma unroll
+    for (int j = 0; j < TILE / 4096; ++j) *(f32x4*)(smem + (NBUF + 7) * TILE + tid * (TILE / 256) + 16 * j) = zero;
   }
   __builtin_amdgcn_s_waitcnt(0);  // retire the Q loads with a wait the compiler can see (and the tiles)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -514,7 +518,7 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
   for (int ks = 0; ks < KS; ++ks) koff_a[ks] = koff[ks] + (int)smem_base;
 #pragma unroll
   for (int db = 0; db < DB; ++db) voff_a[db] = voff[db] + (int)smem_base + NBUF * TILE;  // from the start of the V ring
-  const unsigned lds_dst_k = __builtin_amdgcn_readfirstlane(smem_base + 2 * wave * 1024);
+  const unsigned lds_dst_k = __builtin_amdgcn_readfirstlane(smem_base + PIECES * wave * 1024);
   const unsigned lds_dst_v = lds_dst_k + NBUF * TILE;
   auto uni = [](unsigned x) { return (unsigned)__builtin_amdgcn_readfirstlane((int)x); };
   const unsigned kh_lo = uni((unsigned)(uintptr_t)k_head), kh_hi = uni((unsigned)((uintptr_t)k_head >> 32));
@@ -537,7 +541,11 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
     unsigned k_left = uni((unsigned)kst.left), v_left = uni((unsigned)vst.left);
     unsigned k_next = uni(smem_base + kListAt + 8 * (kst.idx + 1)), v_next = uni(smem_base + kListAt + 8 * (vst.idx + 1));
     const unsigned asm_n = uni((unsigned)N);
+    if constexpr (D == 128) {
 #include "ringattn_walk64_loop.inc"
+    } else {
+#include "ringattn_walk64_loop_d64.inc"
+    }
   } else {
     for (int u = 0; u <= N; ++u) general(u);
   }
@@ -600,32 +608,41 @@ __global__ __launch_bounds__(256, 1) void ring_walk64_kernel(const BlockArgs a) 
     }
   }
   }  // passes
-  if (!KEEP && a.mode == kBlockPartialsMerged) {  // this workgroup's rows over the partials it has just written
-    if (all_items <= kStagedMergeMaxParts)
-      merge_rows_staged<DT, HP>(a, seg, bh, qt, smem, smem_base);
-    else
-      merge_job_rows<DT, D, HP, BM, 64 * WAVES>(a.o_part, a.lse_part, a.out, a.lse, a.items, seg, bh, qt, a.S,
-                                                (lds_float*)(__attribute__((address_space(3))) void*)smem);
+  if constexpr (!KEEP) {
+    if (a.mode == kBlockPartialsMerged) {  // this workgroup's rows over the partials it has just written
+      if (all_items <= kStagedMergeMaxParts)
+        merge_rows_staged<DT, HP>(a, seg, bh, qt, smem, smem_base);
+      else
+        merge_job_rows<DT, D, HP, BM, 64 * WAVES>(a.o_part, a.lse_part, a.out, a.lse, a.items, seg, bh, qt, a.S,
+                                                  (lds_float*)(__attribute__((address_space(3))) void*)smem);
+    }
   }
 }
 
-hipError_t launch_walk64(const BlockArgs& a, int dtype, hipStream_t stream) {
+hipError_t launch_walk64(const BlockArgs& a, int dtype, int dim, hipStream_t stream) {
   if (a.n_segs <= 0) return hipSuccess;
   const int q_tiles = a.q_tiles_max;
   const int64_t groups = (int64_t)a.n_segs * a.BH;
   const int64_t blocks = (a.groups ? (int64_t)a.groups_per_xcd : (groups + 7) / 8) * 8 * q_tiles;
   if (q_tiles <= 0 || blocks > INT32_MAX) return hipErrorInvalidValue;
   if (a.mode != kBlockCarryState && a.mode != kBlockPartials && a.mode != kBlockPartialsMerged) return hipErrorInvalidValue;
+  if (dtype != 0 && dtype != 1) return hipErrorInvalidValue;
   const unsigned grid = (unsigned)blocks;
-#define RA_LAUNCH_WALK64(DT_)                                                                       \
-  do {                                                                                             \
-    if (a.mode == kBlockCarryState) ring_walk64_kernel<DT_, true, false><<<grid, 256, 0, stream>>>(a);  \
-    else if (a.half_partials) ring_walk64_kernel<DT_, false, true><<<grid, 256, 0, stream>>>(a);        \
-    else ring_walk64_kernel<DT_, false, false><<<grid, 256, 0, stream>>>(a);                            \
+  if (dim == 64) {  // state carried only
+    if (a.mode != kBlockCarryState) return hipErrorInvalidValue;
+    if (dtype == 0) ring_walk64_kernel<0, 64, true, false><<<grid, 256, 0, stream>>>(a);
+    else ring_walk64_kernel<1, 64, true, false><<<grid, 256, 0, stream>>>(a);
+    return hipGetLastError();
+  }
+  if (dim != 128) return hipErrorInvalidValue;
+#define RA_LAUNCH_WALK64(DT_)                                                                            \
+  do {                                                                                                  \
+    if (a.mode == kBlockCarryState) ring_walk64_kernel<DT_, 128, true, false><<<grid, 256, 0, stream>>>(a);  \
+    else if (a.half_partials) ring_walk64_kernel<DT_, 128, false, true><<<grid, 256, 0, stream>>>(a);        \
+    else ring_walk64_kernel<DT_, 128, false, false><<<grid, 256, 0, stream>>>(a);                            \
   } while (0)
   if (dtype == 0) RA_LAUNCH_WALK64(0);
-  else if (dtype == 1) RA_LAUNCH_WALK64(1);
-  else return hipErrorInvalidValue;
+  else RA_LAUNCH_WALK64(1);
 #undef RA_LAUNCH_WALK64
   return hipGetLastError();
 }

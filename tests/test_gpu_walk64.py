@@ -41,6 +41,9 @@ def rising_logits(w, slope, period=0):
     (Workload("saw_nc", 1, 3, 128, 3, 768, "fp16", 44, False), 0.4, 300),
     # steep enough for the exponentials to overflow to infinity against a stale reference
     (Workload("steep_c", 1, 1, 128, 2, 1024, "bf16", 45, True), 4.0, 0),
+    # the d = 64 instantiation (half the MFMAs per tile, 4 KB tiles)
+    (Workload("rise64_c", 1, 2, 64, 4, 1024, "bf16", 46, True), 0.2, 0),
+    (Workload("saw64_nc", 2, 1, 64, 3, 768, "fp16", 47, False), 0.3, 300),
 ], ids=lambda x: x.name if isinstance(x, Workload) else None)
 def test_reference_moves_inside_the_hand_scheduled_loop(oracle, w, slope, period):
     q, k, v = rising_logits(w, slope, period)
@@ -57,6 +60,10 @@ def test_reference_moves_inside_the_hand_scheduled_loop(oracle, w, slope, period
     Workload("w_big", 1, 2, 128, 2, 1024, "fp16", 55, False, sigma_qk=3.0),
     Workload("w_tiny", 1, 2, 128, 1, 128, "bf16", 56, True),       # half a q tile: two waves own no row at all
     Workload("w_short", 2, 1, 128, 2, 160, "fp16", 57, False),     # heads shorter than what the load streams run ahead
+    Workload("w64_nc", 2, 3, 64, 4, 512, "fp16", 58, False),       # d = 64
+    Workload("w64_c", 1, 4, 64, 8, 256, "bf16", 59, True),
+    Workload("w64_tiny", 1, 2, 64, 1, 128, "fp16", 60, True),
+    Workload("w64_big", 1, 2, 64, 2, 1024, "fp16", 61, False, sigma_qk=3.0),
 ], ids=lambda w: w.name)
 def test_both_kernels_agree(oracle, w, monkeypatch):
     """The same forward with and without RINGATTN_WIDE=0 (which keeps it on ring_walk_kernel): both against the oracle,
@@ -224,9 +231,10 @@ def test_wide_partials_in_row_major_and_rank_local_buffers(monkeypatch):
 
 def test_random_wide_plans_against_oracle(oracle, monkeypatch):
     """A seeded sweep over the shapes ring_walk64_kernel takes: 1 to 8 ranks of 128 to 1024 tokens each (multiples of
-    32, unequal), batch, grouped heads, both types, the causal mask in both layouts, an explicit scale, graph replay, the
-    state carried or per-step partials (on this kernel: RINGATTN_WIDE_PARTIALS=1).  Every plan must report this kernel;
-    up to 3000 rows of each (the first and the last q tile of a head, chunk edges, random ones) against the oracle."""
+    32, unequal), batch, grouped heads, both head dimensions and types, the causal mask in both layouts, an explicit scale,
+    graph replay, the state carried or per-step partials (on this kernel at d = 128: RINGATTN_WIDE_PARTIALS=1).  Every plan
+    must report this kernel (d = 64 with per-step partials: the other one); up to 3000 rows of each (the first and the last
+    q tile of a head, chunk edges, random ones) against the oracle."""
     monkeypatch.delenv("RINGATTN_WIDE", raising=False)
     monkeypatch.setenv("RINGATTN_WIDE_PARTIALS", "1")
     rng = np.random.default_rng(4242)
@@ -238,25 +246,26 @@ def test_random_wide_plans_against_oracle(oracle, monkeypatch):
         if zigzag:
             lens = [64 * max(4, c // 64) for c in lens]      # both halves of a rank: multiples of 32, at least 128
         dtype = str(rng.choice(["fp16", "bf16"]))
+        d = 64 if case % 4 == 1 else 128
         B, hkv, group = int(rng.integers(1, 3)), int(rng.integers(1, 3)), int(rng.integers(1, 3))
         H, S = hkv * group, sum(lens)
         scale = float(rng.choice([0.0, 0.0, 0.05]))
         graph = bool(rng.integers(0, 2))
         steps_apart = case % 3 == 2
-        tag = (f"case {case}: P={P} lens={lens} B={B} H={H} hkv={hkv} {dtype} causal={causal} zigzag={zigzag} "
+        tag = (f"case {case}: P={P} lens={lens} B={B} H={H} hkv={hkv} d={d} {dtype} causal={causal} zigzag={zigzag} "
                f"scale={scale} graph={graph} step_partials={steps_apart}")
         print(tag, flush=True)
-        w = Workload("wide_rand", B, H, 128, 1, S, dtype, 3000 + case, causal)
+        w = Workload("wide_rand", B, H, d, 1, S, dtype, 3000 + case, causal)
         q, _, _ = api.make_qkv_bits(w)
-        _, k, v = api.make_qkv_bits(Workload("wide_rand_kv", B, hkv, 128, 1, S, dtype, 4000 + case, causal))
+        _, k, v = api.make_qkv_bits(Workload("wide_rand_kv", B, hkv, d, 1, S, dtype, 4000 + case, causal))
         order = api.zigzag_order(lens) if zigzag else np.arange(S)
         inv = torch.from_numpy(np.argsort(order)).cuda()
         qd, kd, vd = (api.bits_to_tensor(np.ascontiguousarray(x[:, :, order]), dtype) for x in (q, k, v))
-        plan = api.RingAttention(P, lens, 128, B, H, dtype, causal, softmax_scale=scale, graph=graph,
+        plan = api.RingAttention(P, lens, d, B, H, dtype, causal, softmax_scale=scale, graph=graph,
                                  kv_heads=hkv if group > 1 else 0, layout="zigzag" if zigzag else "contiguous",
                                  step_partials=steps_apart)
         try:
-            assert plan.forward_kernel() == "ring_walk64_kernel", tag
+            assert plan.forward_kernel() == ("ring_walk_kernel" if d == 64 and steps_apart else "ring_walk64_kernel"), tag
             out, lse = plan.forward(qd, kd, vd)
             if graph:
                 out2, lse2 = plan.forward(qd, kd, vd, torch.empty_like(out), torch.empty_like(lse))

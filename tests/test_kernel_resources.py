@@ -105,10 +105,12 @@ def test_walk64_kernel_runs_one_wave_per_simd(tmp_path):
     is inline assembly)."""
     asm, usage = compile_to_asm("ringattn_walk64.hip", tmp_path / "walk64.s")
     kernels = {n: u for n, u in usage.items() if "ring_walk64_kernel" in n}
-    assert len(kernels) == 6                                  # fp16, bf16 x state carried, fp32 partials, fp16 partials
+    # fp16, bf16 x (d = 128: state carried, fp32 partials, fp16 partials; d = 64: state carried)
+    assert len(kernels) == 8
     for n, u in kernels.items():
+        d64 = "ELi64E" in n
         assert u["Occupancy [waves/SIMD]"] == 1, (n, u)
-        assert u["LDS Size [bytes/block]"] == 2 * 8 * 8192 + 8 * (64 + 4), (n, u)
+        assert u["LDS Size [bytes/block]"] == 2 * 8 * (4096 if d64 else 8192) + 8 * (64 + 4), (n, u)
         # the plain-code path of waves with a single score tile, and the code between the passes of the instantiations
         # that emit a partial per chunk
         assert u["ScratchSize [bytes/lane]"] <= (128 if "ELb1ELb0EE" in n else 448), (n, u)
@@ -116,7 +118,7 @@ def test_walk64_kernel_runs_one_wave_per_simd(tmp_path):
         body = asm[start:asm.index(".amdhsa_kernel " + n, start)]
         blocks = body.split(";;#ASMSTART")[1:]
         loop = max((b.split(";;#ASMEND")[0] for b in blocks), key=len)
-        assert loop.count("v_mfma_f32_32x32x16") >= 8 * 32    # eight unrolled iterations of 32 MFMAs, and the tails
+        assert loop.count("v_mfma_f32_32x32x16") >= 8 * (16 if d64 else 32)    # eight unrolled iterations of 32 (16) MFMAs, and the tails
         assert "scratch_" not in loop
 
 

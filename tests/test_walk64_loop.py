@@ -1,4 +1,5 @@
-"""The hand-scheduled loop of ring_walk64_kernel (ringattention_amd/csrc/gen_walk64_loop.py -> ringattn_walk64_loop.inc):
+"""The hand-scheduled loop of ring_walk64_kernel (ringattention_amd/csrc/gen_walk64_loop.py -> ringattn_walk64_loop.inc
+for d = 128, ringattn_walk64_loop_d64.inc for d = 64):
 the committed file is what the generator writes, and the instruction stream it writes keeps the promises the hardware
 does not check -- every MFMA finds its LDS fragments returned (the s_waitcnt lgkmcnt counts are derived from the order
 of the reads), nothing reads a score tile too soon after the MFMA that wrote it, and an iteration holds the work it
@@ -22,9 +23,10 @@ def gen():
     return mod
 
 
-def test_committed_loop_is_what_the_generator_writes(gen):
-    with open(os.path.join(CSRC, "ringattn_walk64_loop.inc")) as f:
-        assert f.read() == gen.render()
+@pytest.mark.parametrize("d", [128, 64])
+def test_committed_loop_is_what_the_generator_writes(gen, d):
+    with open(os.path.join(CSRC, gen.FILES[d])) as f:
+        assert f.read() == gen.render(d)
 
 
 def regs(token):
@@ -44,23 +46,26 @@ def operands(line):
     return op, [t.strip() for t in rest.split(",")] if rest else []
 
 
+@pytest.mark.parametrize("d", [128, 64])
 @pytest.mark.parametrize("dtype_ops", [("v_mfma_f32_32x32x16_f16", "v_cvt_pk_f16_f32"), ("v_mfma_f32_32x32x16_bf16", "v_cvt_pk_bf16_f32")])
-def test_steady_iterations_hold_their_work_and_wait_for_their_fragments(gen, dtype_ops):
+def test_steady_iterations_hold_their_work_and_wait_for_their_fragments(gen, dtype_ops, d):
     mfma, cvt = dtype_ops
+    gen.configure(d)
+    preread = min(gen.PREREAD, gen.KS)
     del gen._sites[:]
     del gen._redo[:]
     for i in range(gen.UNROLL):
         lines = gen.iteration(i, mfma, cvt)
         ops = [operands(l)[0] for l in lines if not l.endswith(":")]
-        assert sum(o == mfma for o in ops) == 32                          # 16 for S(u+1) = K Q^T, 16 for O += P V
-        assert sum(o.startswith("ds_read") for o in ops) == 24            # 8 K fragments, 16 halves of V^T fragments
-        assert sum(o == "global_load_lds_dwordx4" for o in ops) == 4      # this wave's two pieces of two tiles
+        assert sum(o == mfma for o in ops) == d // 4                      # half for S(u+1) = K Q^T, half for O += P V
+        assert sum(o.startswith("ds_read") for o in ops) == 3 * d // 16   # d / 16 K fragments, d / 8 halves of V^T fragments
+        assert sum(o == "global_load_lds_dwordx4" for o in ops) == d // 32   # this wave's pieces of two tiles
         assert sum(o == "v_exp_f32" for o in ops) == 32                   # one exponential per score
         assert sum(o == "s_barrier" for o in ops) == (1 if i % 2 == 0 else 0)
         assert not any(o.startswith(("scratch_", "buffer_", "flat_")) for o in ops)
         # LDS reads return in order: replay the queue, and require every fragment register an MFMA reads to be back
         outstanding = []                  # reads not yet waited for, oldest first: the registers each one writes
-        for ks in range(gen.PREREAD):     # (the first K fragments were read ahead by the iteration before)
+        for ks in range(preread):         # (the first K fragments were read ahead by the iteration before)
             outstanding.append({("v", r) for r in regs(gen.KF(ks))[1]})
         last_writer = {}                  # score register -> index of the MFMA that wrote it
         n = 0
@@ -91,10 +96,13 @@ def test_steady_iterations_hold_their_work_and_wait_for_their_fragments(gen, dty
                         if f == "v" and r in last_writer:
                             assert n - last_writer[r] > 11, (i, line)
         # what is still out at the end are the K fragments read ahead for the next iteration
-        assert len(outstanding) == gen.PREREAD
+        assert len(outstanding) == preread
+    gen.configure(128)
 
 
-def test_loop_text_has_every_exit_and_no_stray_label(gen):
+@pytest.mark.parametrize("d", [128, 64])
+def test_loop_text_has_every_exit_and_no_stray_label(gen, d):
+    gen.configure(d)
     lines = gen.loop_text("v_mfma_f32_32x32x16_bf16", "v_cvt_pk_bf16_f32")
     labels = [l[:-1] for l in lines if l.endswith(":")]
     assert len(labels) == len(set(labels))
@@ -108,3 +116,4 @@ def test_loop_text_has_every_exit_and_no_stray_label(gen):
         m = re.match(r"s_c?branch\w*\s+(\d+)([fb])$", l)
         if m:
             assert (pos[m.group(1)] > k) == (m.group(2) == "f"), l
+    gen.configure(128)
