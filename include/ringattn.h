@@ -237,9 +237,10 @@ int ringattn_plan_work_items(const ringattn_plan* plan, int step, ringattn_work_
 int ringattn_plan_launch_times(ringattn_plan* plan, float* ms, int capacity, int* n_out);
 
 /*
- * Name of the kernel ringattn_fwd launches for this plan, for reading kernel traces: "ring_walk64_kernel" (d = 128,
- * carried softmax state, every KV range a multiple of 32 keys and at least 128, at least 512 rows per head, and
- * RINGATTN_WIDE=0 not set in the environment) or "ring_walk_kernel".  Both are restatements of the reference's one
+ * Name of the kernel ringattn_fwd launches for this plan, for reading kernel traces: "ring_walk64_kernel" (every KV
+ * range a multiple of 32 keys and at least 128; with RINGATTN_FLAG_STEP_PARTIALS only at d = 128 in causal plans with at
+ * least 2048 keys per chunk; RINGATTN_WIDE=0, RINGATTN_WIDE_D64=0 and RINGATTN_WIDE_PARTIALS=0 / 1 in the environment
+ * override) or "ring_walk_kernel".  Both are restatements of the reference's one
  * kernel (csrc/ring_attention.cu:398-666) with its tiling (csrc/kernel_traits.h:11-177) replaced; they differ in how
  * the 256 query rows of a workgroup are laid out over waves (64 rows per wave at one wave per SIMD, or 32 rows per
  * wave at two).  NULL for an invalid plan.
