@@ -34,10 +34,10 @@ PEAK_HBM_GBS = 8000.0
 # (bytes, summary under profiles/, kernel, kernel_source_id(kernel) when it was measured).  The figure is only printed
 # while the forward still runs that kernel and its source is still the one that was profiled.
 MEASURED_TRAFFIC = {
-    "cfg4": (2259e6, "profiles/ring_walk64_kernel_cfg4.md", "ring_walk64_kernel", "69c40bef835e5420"),
-    "cfg3": (2408e6, "profiles/ring_walk64_kernel_other_workloads.md", "ring_walk64_kernel", "69c40bef835e5420"),
-    "cfg5": (50670e6, "profiles/ring_walk64_kernel_other_workloads.md", "ring_walk64_kernel", "69c40bef835e5420"),
-    "cfg2": (34.3e6, "profiles/ring_walk64_kernel_other_workloads.md", "ring_walk64_kernel", "69c40bef835e5420"),
+    "cfg4": (2243e6, "profiles/ring_walk64_kernel_cfg4.md", "ring_walk64_kernel", "4f2da51b8ee24e2d"),
+    "cfg3": (2328e6, "profiles/ring_walk64_kernel_other_workloads.md", "ring_walk64_kernel", "4f2da51b8ee24e2d"),
+    "cfg5": (48980e6, "profiles/ring_walk64_kernel_other_workloads.md", "ring_walk64_kernel", "4f2da51b8ee24e2d"),
+    "cfg2": (34.3e6, "profiles/ring_walk64_kernel_other_workloads.md", "ring_walk64_kernel", "4f2da51b8ee24e2d"),
 }
 KERNEL_SOURCES = {
     "ring_walk64_kernel": ("ringattn_walk64.hip", "ringattn_walk64_loop.inc", "ringattn_walk64_loop_d64.inc", "ringattn_device.h"),

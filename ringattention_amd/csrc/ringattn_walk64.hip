@@ -3,7 +3,7 @@
 //   ring_walk64_kernel : the forward of ring_walk_kernel (ringattn_walk.hip; the reference's CTA
 //       that walks its ring steps with max / sum / acc-O in registers,
 //       csrc/ring_attention.cu:439-443,456-620, epilogue :621-664; or, chunk by chunk, with a partial
-//       (O, LSE) per ring step and their merge at the end) for d = 128, laid out for ONE wave
+//       (O, LSE) per ring step and their merge at the end), laid out for ONE wave
 //       per SIMD: a workgroup of FOUR waves owns the same 256 query rows, each wave two 32-query
 //       blocks.  Every K fragment and every V^T fragment read from LDS then feeds two MFMAs (one per
 //       block) instead of one: half the LDS fragment traffic per MFMA.  With 512 registers per wave
@@ -19,8 +19,9 @@
 //       One wave per SIMD has nobody to wait behind, so nothing may be waited for: the K and V rings are eight
 //       tiles deep (128 KB of LDS) and a tile is loaded four or more iterations before the barrier that hands it
 //       over (s_waitcnt vmcnt(12): the loads of the last three iterations stay in flight).
-//       Shapes it takes: every KV range a multiple of 32 keys and at least 128 (the host checks); anything else
-//       runs ring_walk_kernel.
+//       Described for d = 128; at d = 64 (state carried only) a tile is 4 KB, an iteration has 16 MFMAs and the
+//       rings take 64 KB.  Shapes it takes: every KV range a multiple of 32 keys and at least 128 (the host checks);
+//       anything else runs ring_walk_kernel.
 #include "ringattn_device.h"
 
 #include <type_traits>
