@@ -210,7 +210,8 @@ def exp_stream(cur, cvt):
         if kind == 0:
             valu.append("v_fma_f32 %s, %s, %s, -%s" % (PX(b, e), Sreg(cur, b, e), S_K2, MS(b)))
         elif kind == 1:
-            valu.append("v_exp_f32 %s, %s" % (PX(b, e), PX(b, e)))
+            op = "v_mov_b32" if _knob('EXPMOV', 0) else "v_exp_f32"   # (timing only: what the transcendental itself costs)
+            valu.append("%s %s, %s" % (op, PX(b, e), PX(b, e)))
         else:
             if e >= 4:
                 first = PX(b, e - 4) if e < 8 else TS(b, e & 3)
